@@ -1,0 +1,241 @@
+// GEMM entry points: C = round(beta*C + relu(alpha * op(A).op(B))).
+// Replaces the {h,s}gemm_{nn,nt,tn}[_vec]_{tile} kernel family selected in
+// NervanaGPU.dot / batched_dot (nervanagpu/nervanagpu.py:820-1105) and the
+// GEMM-only C interface (kernels/C_interface/nervana_c_api.h:31-128).
+#include "gemm_core.h"
+
+#include <algorithm>
+
+namespace ng {
+
+struct GemmArgs {
+    int trans_a, trans_b;
+    int m, n, k;
+    const void* A; int lda;
+    const void* B; int ldb;
+    void* C; int ldc;
+    float alpha, beta;
+    unsigned flags, seed, rng_stream;
+    int batch_grid; long ldaz, ldbz, ldcz; int batch_loops;
+    void* ws; size_t ws_bytes;
+    hipStream_t stream;
+};
+
+struct TileChoice { int bm, bn, bk, threads; };
+
+static int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// how many slices to cut the contraction into so that the grid fills the chip
+static int choose_splits(int out_tiles, int total_k_tiles, size_t slice_bytes, size_t ws_bytes)
+{
+    const int cus = device_cu_count();
+    if (out_tiles >= cus || total_k_tiles < 8) return 1;
+    int splits = ceil_div(2 * cus, out_tiles);
+    splits = std::min(splits, total_k_tiles / 4);
+    if (slice_bytes) splits = (int)std::min<size_t>((size_t)splits, ws_bytes / slice_bytes);
+    // every slice must own at least one tile
+    while (splits > 1 && (splits - 1) * ceil_div(total_k_tiles, splits) >= total_k_tiles) splits--;
+    return std::max(splits, 1);
+}
+
+template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, bool VEC>
+static int launch_gemm(const GemmArgs& g, unsigned sr_bits)
+{
+    CoreShape s;
+    s.m = g.m; s.n = g.n;
+    s.k_tiles = ceil_div(g.k, BK);
+    s.passes = g.batch_loops;
+    s.tiles_m = ceil_div(g.m, BM);
+    s.tiles_n = ceil_div(g.n, BN);
+    const int zcount = g.batch_grid;
+    const int out_tiles = s.tiles_m * s.tiles_n * zcount;
+    const size_t slice_bytes = (size_t)zcount * g.m * g.n * sizeof(float);
+    s.splits = g.ws ? choose_splits(out_tiles, s.passes * s.k_tiles, slice_bytes, g.ws_bytes) : 1;
+
+    DenseLoader<T, LA, VEC> al{(const T*)g.A, g.ldaz, g.lda, g.m, g.k};
+    DenseLoader<T, LB, VEC> bl{(const T*)g.B, g.ldbz, g.ldb, g.n, g.k};
+    ScaleStoreEpilogue<T> epi{(T*)g.C, g.ldcz, g.ldc, g.m, g.n, g.alpha, g.beta,
+                              (g.flags & NG_FLAG_RELU) ? 1u : 0u, sr_bits, g.seed, g.rng_stream,
+                              (((uintptr_t)g.C & 15) == 0 && g.ldc % 8 == 0 && g.ldcz % 8 == 0 && g.n % 8 == 0) ? 1u : 0u};
+
+    dim3 grid(s.tiles_m * s.tiles_n, s.splits, zcount);
+    dim3 block(WM * WN * 64);
+    if (s.splits == 1) {
+        hipLaunchKernelGGL((mfma_gemm_kernel<T, BM, BN, BK, WM, WN, LA, LB, DenseLoader<T, LA, VEC>,
+                                             DenseLoader<T, LB, VEC>, ScaleStoreEpilogue<T>>),
+                           grid, block, 0, g.stream, al, bl, epi, s);
+        NG_CHECK_LAUNCH("gemm kernel");
+    } else {
+        PartialEpilogue pe{(float*)g.ws, g.m, g.n, zcount, (g.n % 8 == 0) ? 1u : 0u};
+        hipLaunchKernelGGL((mfma_gemm_kernel<T, BM, BN, BK, WM, WN, LA, LB, DenseLoader<T, LA, VEC>,
+                                             DenseLoader<T, LB, VEC>, PartialEpilogue>),
+                           grid, block, 0, g.stream, al, bl, pe, s);
+        NG_CHECK_LAUNCH("gemm split kernel");
+        const long total = (long)zcount * g.m * g.n;
+        const int blocks = (int)std::min<long>((total + 255) / 256, 8192);
+        hipLaunchKernelGGL((splitk_reduce_kernel<T, ScaleStoreEpilogue<T>>), dim3(blocks), dim3(256), 0, g.stream,
+                           (const float*)g.ws, s.splits, zcount, g.m, g.n, epi);
+        NG_CHECK_LAUNCH("gemm split reduce");
+    }
+    return 0;
+}
+
+template <typename T, int BM, int BN, int BK, int WM, int WN, bool VEC>
+static int launch_layout(const GemmArgs& g, unsigned sr_bits)
+{
+    if (!g.trans_a && !g.trans_b) return launch_gemm<T, BM, BN, BK, WM, WN, KC, MC, VEC>(g, sr_bits);
+    if (!g.trans_a && g.trans_b)  return launch_gemm<T, BM, BN, BK, WM, WN, KC, KC, VEC>(g, sr_bits);
+    return launch_gemm<T, BM, BN, BK, WM, WN, MC, MC, VEC>(g, sr_bits);
+}
+
+template <typename T>
+static bool operands_vectorizable(const GemmArgs& g)
+{
+    constexpr int EPC = Elem<T>::EPC;
+    auto ok = [&](const void* p, int ld, long ldz, int contiguous_extent) {
+        return ((uintptr_t)p & 15) == 0 && ld % EPC == 0 && ldz % EPC == 0 && contiguous_extent % EPC == 0;
+    };
+    const bool a = ok(g.A, g.lda, g.ldaz, g.trans_a ? g.m : g.k);
+    const bool b = ok(g.B, g.ldb, g.ldbz, g.trans_b ? g.k : g.n);
+    return a && b;
+}
+
+template <typename T> static int dispatch(const GemmArgs& g, unsigned sr_bits);
+
+template <>
+int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
+{
+    const bool vec = operands_vectorizable<_Float16>(g);
+    const long big_tiles = (long)ceil_div(g.m, 256) * ceil_div(g.n, 256) * g.batch_grid;
+    const bool large = g.m >= 256 && g.n >= 256 && big_tiles >= device_cu_count() / 2;
+    if (large) {
+        return vec ? launch_layout<_Float16, 256, 256, 32, 2, 2, true>(g, sr_bits)
+                   : launch_layout<_Float16, 256, 256, 32, 2, 2, false>(g, sr_bits);
+    }
+    return vec ? launch_layout<_Float16, 128, 128, 32, 2, 2, true>(g, sr_bits)
+               : launch_layout<_Float16, 128, 128, 32, 2, 2, false>(g, sr_bits);
+}
+
+template <>
+int dispatch<float>(const GemmArgs& g, unsigned sr_bits)
+{
+    const bool vec = operands_vectorizable<float>(g);
+    return vec ? launch_layout<float, 128, 128, 16, 2, 2, true>(g, sr_bits)
+               : launch_layout<float, 128, 128, 16, 2, 2, false>(g, sr_bits);
+}
+
+static int check_args(const GemmArgs& g, int dtype)
+{
+    if (dtype != NG_F16 && dtype != NG_F32) return fail(-20, "ng_gemm: only floating point dot is supported");
+    if (g.trans_a && g.trans_b) return fail(-21, "ng_gemm: op \"tt\" is not supported");
+    if (g.m < 0 || g.n < 0 || g.k < 0) return fail(-22, "ng_gemm: negative extent");
+    if (g.batch_grid < 1 || g.batch_loops < 1) return fail(-23, "ng_gemm: batch_grid and batch_loops must be >= 1");
+    if (g.batch_grid > 1 && g.batch_loops > 1) return fail(-24, "ng_gemm: batch_grid and batch_loops are exclusive");
+    if (g.m && g.n && (!g.C || (g.k && (!g.A || !g.B)))) return fail(-25, "ng_gemm: null operand");
+    const int a_cols = g.trans_a ? g.m : g.k, b_cols = g.trans_b ? g.k : g.n;
+    if (g.lda < a_cols || g.ldb < b_cols || g.ldc < g.n) return fail(-26, "ng_gemm: leading dimension smaller than row length");
+    if ((long)g.batch_grid * g.m * g.n >= (1L << 32)) return fail(-27, "ng_gemm: output larger than 2^32 elements");
+    return 0;
+}
+
+static unsigned sr_bits_of(unsigned flags, int dtype)
+{
+    if (!(flags & NG_FLAG_SR)) return 0;
+    unsigned bits = flags >> 16;
+    if (bits == 0) bits = 10;
+    const unsigned cap = (dtype == NG_F16) ? 10u : 15u;
+    return std::max(1u, std::min(bits, cap));
+}
+
+}  // namespace ng
+
+using namespace ng;
+
+extern "C" {
+
+size_t ng_gemm_workspace_bytes(int dtype, int trans_a, int trans_b, int m, int n, int k,
+                               int batch_grid, int batch_loops)
+{
+    (void)trans_a; (void)trans_b;
+    const int bk = (dtype == NG_F16) ? 32 : 16;
+    const int bt = 128;
+    const int out_tiles = ceil_div(m, bt) * ceil_div(n, bt) * batch_grid;
+    const int total_k = ceil_div(k, bk) * batch_loops;
+    const int splits = choose_splits(out_tiles, total_k, 0, 0);
+    if (splits <= 1) return 0;
+    return (size_t)splits * batch_grid * m * n * sizeof(float);
+}
+
+int ng_gemm(int dtype, int trans_a, int trans_b, int m, int n, int k,
+            const void* A, int lda, const void* B, int ldb, void* C, int ldc,
+            float alpha, float beta, unsigned flags,
+            unsigned seed, unsigned rng_stream,
+            int batch_grid, long ldaz, long ldbz, long ldcz, int batch_loops,
+            void* workspace, size_t workspace_bytes, void* stream)
+{
+    GemmArgs g{trans_a, trans_b, m, n, k, A, lda, B, ldb, C, ldc, alpha, beta, flags, seed, rng_stream,
+               batch_grid, ldaz, ldbz, ldcz, batch_loops, workspace, workspace_bytes, (hipStream_t)stream};
+    int rc = check_args(g, dtype);
+    if (rc) return rc;
+    if (m == 0 || n == 0) return 0;
+    const unsigned sr_bits = sr_bits_of(flags, dtype);
+    return dtype == NG_F16 ? dispatch<_Float16>(g, sr_bits) : dispatch<float>(g, sr_bits);
+}
+
+// ---- GEMM-only C interface (kernels/C_interface/nervana_c_api.h) -----------
+
+bool nervana_loadKernels(const char* /*base_path*/)
+{
+    // kernels are linked into this library; select the current device
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+    return ng_init(dev) == 0;
+}
+
+bool nervana_unloadKernels(void) { return true; }
+
+size_t nervana_randStateSizeBytes(void) { return 2048 * 32 * sizeof(unsigned); }
+
+static bool c_gemm(int dtype, void* A, void* B, void* C, bool a_t, bool b_t, int m, int n, int k,
+                   int lda, int ldb, int ldc, float alpha, float beta, bool sr, bool relu, void* stream)
+{
+    unsigned flags = (sr ? (NG_FLAG_SR | (10u << 16)) : 0u) | (relu ? NG_FLAG_RELU : 0u);
+    static unsigned call_counter = 0;
+    int rc = ng_gemm(dtype, a_t, b_t, m, n, k, A, lda, B, ldb, C, ldc, alpha, beta, flags,
+                     0u, sr ? ++call_counter : 0u, 1, 0, 0, 0, 1, nullptr, 0, stream);
+    if (rc) fprintf(stderr, "nervana gemm: %s\n", ng_last_error());
+    return rc == 0;
+}
+
+bool nervana_sgemm(float* A, float* B, float* C, bool a_t, bool b_t, int m, int n, int k,
+                   int lda, int ldb, int ldc, float alpha, float beta, unsigned int* /*rand_state*/,
+                   bool stochastic_round, bool apply_relu, void* stream, int /*grid*/)
+{
+    return c_gemm(NG_F32, A, B, C, a_t, b_t, m, n, k, lda, ldb, ldc, alpha, beta, stochastic_round, apply_relu, stream);
+}
+
+bool nervana_hgemm(short* A, short* B, short* C, bool a_t, bool b_t, int m, int n, int k,
+                   int lda, int ldb, int ldc, float alpha, float beta, unsigned int* /*rand_state*/,
+                   bool stochastic_round, bool apply_relu, void* stream, int /*grid*/)
+{
+    return c_gemm(NG_F16, A, B, C, a_t, b_t, m, n, k, lda, ldb, ldc, alpha, beta, stochastic_round, apply_relu, stream);
+}
+
+// column-major C(m,n) = op(A).op(B) is the row-major product C^T(n,m) = op(B)^T.op(A)^T
+bool nervana_sgemm_colmajor(float* A, float* B, float* C, bool a_t, bool b_t, int m, int n, int k,
+                            int lda, int ldb, int ldc, float alpha, float beta, unsigned int* rand_state,
+                            bool stochastic_round, bool apply_relu, void* stream, int grid)
+{
+    return nervana_sgemm(B, A, C, b_t, a_t, n, m, k, ldb, lda, ldc, alpha, beta, rand_state,
+                         stochastic_round, apply_relu, stream, grid);
+}
+
+bool nervana_hgemm_colmajor(short* A, short* B, short* C, bool a_t, bool b_t, int m, int n, int k,
+                            int lda, int ldb, int ldc, float alpha, float beta, unsigned int* rand_state,
+                            bool stochastic_round, bool apply_relu, void* stream, int grid)
+{
+    return nervana_hgemm(B, A, C, b_t, a_t, n, m, k, ldb, lda, ldc, alpha, beta, rand_state,
+                         stochastic_round, apply_relu, stream, grid);
+}
+
+}  // extern "C"
