@@ -140,22 +140,30 @@ typedef struct ng_conv_params {
     int str_d, str_h, str_w;
 } ng_conv_params;
 
-/* scratch bytes needed by the three conv ops for this geometry (filter
- * re-layout for bprop, split partial sums for update) */
-size_t ng_conv_workspace_bytes(const ng_conv_params* p, int dtype);
+/* ConvLayer.__init__ precomputes every launch constant once per layer
+ * (nervanagpu/layers.py:281-481); the plan is the counterpart: it owns the small
+ * device-side tap tables of one geometry.  dtype is the storage type of the
+ * filters and of the fprop/bprop outputs (NG_F16 or NG_F32). */
+int ng_conv_plan_create(const ng_conv_params* p, int dtype, void** plan);
+int ng_conv_plan_destroy(void* plan);
+/* scratch bytes the three conv ops may use for this plan (filter re-layout for
+ * bprop, split partial sums for update); the reference keeps one shared scratch
+ * buffer for the same two purposes (nervanagpu/nervanagpu.py:686-698) */
+size_t ng_conv_plan_workspace_bytes(const void* plan);
 /* O = round(relu?(alpha * conv(I, F))).  in_dtype may be NG_U8/NG_I8 with
- * dtype NG_F16/NG_F32 filters and output: the bytes are converted exactly on
- * load (declared at README.md:37, stubs kernels/cu/hconv_fprop_u8_K64_N64.cu). */
-int ng_conv_fprop(const ng_conv_params* p, int dtype, int in_dtype,
+ * NG_F16 filters and output: the bytes are converted exactly on load (declared
+ * at README.md:37, stubs kernels/cu/hconv_fprop_u8_K64_N64.cu:19-40). */
+int ng_conv_fprop(const void* plan, int in_dtype,
                   const void* I, const void* F, void* O, float alpha, unsigned flags,
                   void* workspace, size_t workspace_bytes, void* stream);
-/* gradI = round(alpha * conv_transpose(E, F)); deterministic gather form */
-int ng_conv_bprop(const ng_conv_params* p, int dtype,
+/* gradI = round(alpha * conv_transpose(E, F)); deterministic gather form, every
+ * element of gradI is written (no zero fill needed) */
+int ng_conv_bprop(const void* plan,
                   const void* F, const void* E, void* gradI, float alpha,
                   void* workspace, size_t workspace_bytes, void* stream);
 /* gradF = round(alpha * sum_{pixels,n} I x E); out_dtype NG_F32 or NG_F16;
  * fp32 accumulation with a fixed-order reduction of the split partial sums */
-int ng_conv_update(const ng_conv_params* p, int dtype, int in_dtype, int out_dtype,
+int ng_conv_update(const void* plan, int in_dtype, int out_dtype,
                    const void* I, const void* E, void* gradF, float alpha,
                    void* workspace, size_t workspace_bytes, void* stream);
 
@@ -175,9 +183,12 @@ int ng_pool_fprop(const ng_pool_params* p, int dtype, int op,
                   const void* I, void* O, void* stream);
 /* gradI is fully written (no zero fill needed); window overlap is resolved by a
  * gather over the windows touching each input element, so the result does not
- * depend on execution order. */
+ * depend on execution order.  Overlapping max pooling keeps one byte per output
+ * element (the argmax slot) in `workspace`. */
+size_t ng_pool_workspace_bytes(const ng_pool_params* p, int dtype, int op);
 int ng_pool_bprop(const ng_pool_params* p, int dtype, int op,
-                  const void* I, const void* E, void* gradI, void* stream);
+                  const void* I, const void* E, void* gradI,
+                  void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- small data-movement helpers ---------------------------------------------
  * transpose / dimShuffle / fp32 convert kernels of nervanagpu/float_ew.py:1325-1428 */

@@ -87,16 +87,19 @@ _SIGNATURES = {
     "nervana_hgemm_colmajor": (c_bool, [c_void_p, c_void_p, c_void_p, c_bool, c_bool, c_int, c_int,
                                         c_int, c_int, c_int, c_int, c_float, c_float, c_void_p,
                                         c_bool, c_bool, c_void_p, c_int]),
-    "ng_conv_workspace_bytes": (c_size_t, [POINTER(ConvParams), c_int]),
-    "ng_conv_fprop": (c_int, [POINTER(ConvParams), c_int, c_int, c_void_p, c_void_p, c_void_p,
+    "ng_conv_plan_create": (c_int, [POINTER(ConvParams), c_int, POINTER(c_void_p)]),
+    "ng_conv_plan_destroy": (c_int, [c_void_p]),
+    "ng_conv_plan_workspace_bytes": (c_size_t, [c_void_p]),
+    "ng_conv_fprop": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                               c_float, c_uint, c_void_p, c_size_t, c_void_p]),
-    "ng_conv_bprop": (c_int, [POINTER(ConvParams), c_int, c_void_p, c_void_p, c_void_p,
+    "ng_conv_bprop": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p,
                               c_float, c_void_p, c_size_t, c_void_p]),
-    "ng_conv_update": (c_int, [POINTER(ConvParams), c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+    "ng_conv_update": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                c_float, c_void_p, c_size_t, c_void_p]),
     "ng_pool_fprop": (c_int, [POINTER(PoolParams), c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "ng_pool_workspace_bytes": (c_size_t, [POINTER(PoolParams), c_int, c_int]),
     "ng_pool_bprop": (c_int, [POINTER(PoolParams), c_int, c_int, c_void_p, c_void_p, c_void_p,
-                              c_void_p]),
+                              c_void_p, c_size_t, c_void_p]),
     "ng_transpose": (c_int, [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "ng_dimshuffle": (c_int, [c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "ng_fp32_convert": (c_int, [c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
@@ -150,13 +153,23 @@ def device_count():
     return n.value if st == 0 else 0
 
 
-def init(device=0):
-    """Lazy device initialisation (replaces `import pycuda.autoinit`)."""
+_default_device = 0
+
+
+def set_default_device(device):
+    """device used by the lazy initialisation (NervanaGPU(device=...))"""
+    global _default_device
+    _default_device = int(device)
+
+
+def init(device=None):
+    """Lazy device initialisation (replaces `import pycuda.autoinit`); raises
+    NervanaGPUError when the library or a gfx950 device is missing."""
     global _initialised_device
+    if device is None:
+        device = _default_device
     if _initialised_device == device:
         return
-    with _lock:
-        pass
     call("ng_init", device)
     _initialised_device = device
 

@@ -152,7 +152,10 @@ struct DenseLoader {
     int      rows;   // extent along r
     int      kdim;   // extent along k (per pass)
 
-    __device__ __forceinline__ uint4_t load(int r, int k, int zb) const
+    typedef int Ctx;   // per-chunk row context: the row index itself
+    __device__ __forceinline__ Ctx prepare(int r) const { return r; }
+
+    __device__ __forceinline__ uint4_t load(const Ctx& r, int k, int zb) const
     {
         constexpr int EPC = Elem<T>::EPC;
         const T* p = base + (long)zb * ldz;
@@ -243,7 +246,10 @@ void mfma_gemm_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % KSTEP == 0, "bad tile shape");
 
     constexpr int STAGE = TA::BYTES + TB::BYTES;
-    constexpr int SMEM_BYTES = 2 * STAGE;
+    constexpr int WTN = BN / WN;                 // columns of a wavefront's sub-tile
+    constexpr int EPITCH = WTN * 4 + 16;         // bytes per staged epilogue row
+    constexpr int EPI_BYTES = 32 * EPITCH;       // epilogue staging per wavefront
+    constexpr int SMEM_BYTES = (2 * STAGE > EPI_BYTES * WM * WN) ? 2 * STAGE : EPI_BYTES * WM * WN;
     __shared__ __attribute__((aligned(16))) char smem[SMEM_BYTES];
 
     const int tid = threadIdx.x;
@@ -270,6 +276,14 @@ void mfma_gemm_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
 #pragma unroll
     for (int i = 0; i < CPT_B; i++) TB::chunk_pos(tid + i * NT, rb_r[i], rb_k[i], rb_off[i]);
 
+    // loaders may precompute per-row state (e.g. the pixel a column belongs to)
+    typename ALoad::Ctx actx[CPT_A];
+    typename BLoad::Ctx bctx[CPT_B];
+#pragma unroll
+    for (int i = 0; i < CPT_A; i++) actx[i] = aload.prepare(m0 + ra_r[i]);
+#pragma unroll
+    for (int i = 0; i < CPT_B; i++) bctx[i] = bload.prepare(n0 + rb_r[i]);
+
     uint4_t ra[CPT_A], rb[CPT_B];
     float16_t acc[TM][TN];
 #pragma unroll
@@ -283,9 +297,9 @@ void mfma_gemm_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
         const int pass = t / s.k_tiles;
         const int k0 = (t - pass * s.k_tiles) * BK;
 #pragma unroll
-        for (int i = 0; i < CPT_A; i++) ra[i] = aload.load(m0 + ra_r[i], k0 + ra_k[i], z + pass);
+        for (int i = 0; i < CPT_A; i++) ra[i] = aload.load(actx[i], k0 + ra_k[i], z + pass);
 #pragma unroll
-        for (int i = 0; i < CPT_B; i++) rb[i] = bload.load(n0 + rb_r[i], k0 + rb_k[i], z + pass);
+        for (int i = 0; i < CPT_B; i++) rb[i] = bload.load(bctx[i], k0 + rb_k[i], z + pass);
     };
     auto sstore = [&](int buf) {
 #pragma unroll
@@ -331,10 +345,6 @@ void mfma_gemm_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     // band of its sub-tile at a time through a private LDS region so that a lane
     // ends up with 8 consecutive columns of one row: the global stores (and the
     // beta*C loads) are then 16-byte accesses covering whole rows.
-    constexpr int WTN = BN / WN;                 // columns of a wavefront's sub-tile
-    constexpr int EPITCH = WTN * 4 + 16;         // bytes per staged row
-    constexpr int EPI_BYTES = 32 * EPITCH;       // per wavefront
-    static_assert(EPI_BYTES * WM * WN <= SMEM_BYTES, "epilogue staging does not fit");
     char* stage = smem + wave * EPI_BYTES;
     __syncthreads();
     EpilogueBands<TM, TN, WTN, EPITCH, 0>::run(acc, stage, lane, m0 + wm * (BM / WM), n0 + wn * WTN, z, split, epi);

@@ -1,0 +1,979 @@
+"""
+Fused elementwise / reduction / broadcast kernels, generated at run time.
+
+Host-side counterpart of the reference's compound-kernel generator
+(nervanagpu/float_ew.py:540-1322): a postfix expression stack is turned into
+ONE kernel that keeps every intermediate in fp32 registers, performs all
+reductions of the expression along one axis, and rounds once on the final
+store (nearest, or stochastic for fp16/fp32 outputs).  Same operator
+vocabulary (op table float_ew.py:464-533), same broadcasting rules
+(:1156-1218), same de-duplication of repeated reductions (:614-647), same
+argmax/argmin tie rule (lower index wins, :519-532).
+
+What is different is the kernel shape, chosen for CDNA4:
+  * the source is HIP, compiled with hiprtc for gfx950 and cached per
+    expression signature;
+  * a workgroup owns one row (the reduced axis) and lanes own 16-byte vectors of
+    consecutive elements whenever the operands are contiguous and aligned;
+  * when the row fits in registers (<= 32 values per lane) every operand is read
+    from memory exactly once and all reduction stages run on the cached
+    registers, so e.g. batch normalisation moves 1 read + 1 write per element
+    instead of 3 reads + 1 write;
+  * reductions are 64-lane butterfly shuffles, LDS is only used to combine
+    wavefronts;
+  * plain contiguous expressions (no reduction / broadcast / transpose / take)
+    run as one flat grid-stride kernel instead of one workgroup per 256 elements;
+  * stochastic rounding draws from a counter-based stream keyed on
+    (seed, launch counter, logical element index), so results are reproducible.
+"""
+import ctypes
+from ctypes import c_float, c_int, c_uint, c_void_p
+
+import numpy as np
+
+from . import _lib
+
+# op name -> (operand count, C expression); {0},{1} are the operands in source order
+_float_ops = {
+    "assign":  (2, None),
+    "add":     (2, "({0} + {1})"),
+    "sub":     (2, "({0} - {1})"),
+    "mul":     (2, "({0} * {1})"),
+    "div":     (2, "({0} / {1})"),
+    "eq":      (2, "(({0} == {1}) ? 1.0f : 0.0f)"),
+    "ne":      (2, "(({0} != {1}) ? 1.0f : 0.0f)"),
+    "lt":      (2, "(({0} <  {1}) ? 1.0f : 0.0f)"),
+    "le":      (2, "(({0} <= {1}) ? 1.0f : 0.0f)"),
+    "gt":      (2, "(({0} >  {1}) ? 1.0f : 0.0f)"),
+    "ge":      (2, "(({0} >= {1}) ? 1.0f : 0.0f)"),
+    "minimum": (2, "fminf({0}, {1})"),
+    "maximum": (2, "fmaxf({0}, {1})"),
+    "pow":     (2, "powf({0}, {1})"),
+    "finite":  (1, "(isfinite({0}) ? 1.0f : 0.0f)"),
+    "neg":     (1, "(-{0})"),
+    "abs":     (1, "fabsf({0})"),
+    "sgn":     (1, "copysignf(1.0f, {0})"),
+    "sqrt":    (1, "sqrtf({0})"),
+    "sqr":     (1, "({0} * {0})"),
+    "exp":     (1, "expf({0})"),
+    "log":     (1, "logf({0})"),
+    "exp2":    (1, "exp2f({0})"),
+    "log2":    (1, "log2f({0})"),
+    "sig":     (1, "(1.0f / (1.0f + expf(-{0})))"),
+    "sig2":    (1, "(1.0f / (1.0f + exp2f(-{0})))"),
+    "tanh":    (1, "tanhf({0})"),
+    "tanh2":   (1, "((exp2f(2.0f * {0}) - 1.0f) / (exp2f(2.0f * {0}) + 1.0f))"),
+    "rand":    (0, None),
+    "onehot":  (0, None),
+}
+
+_reduction_ops = ("sum", "max", "min", "argmax", "argmin")
+
+_ew_types = {
+    "f4": ("float", None),
+    "f2": ("_Float16", None),
+    "i4": ("int", (-2147483648.0, 2147483520.0)),
+    "u4": ("unsigned int", (0.0, 4294967040.0)),
+    "i2": ("short", (-32768.0, 32767.0)),
+    "u2": ("unsigned short", (0.0, 65535.0)),
+    "i1": ("signed char", (-128.0, 127.0)),
+    "u1": ("unsigned char", (0.0, 255.0)),
+}
+
+MAX_CACHED_PER_LANE = 32     # fp32 registers per operand kept resident per lane
+MAX_THREADS = 1024
+
+
+def _contiguous_strides(shape):
+    if not shape:
+        return ()
+    strides = [1]
+    for s in shape[:0:-1]:
+        strides.append(strides[-1] * s)
+    return tuple(strides[::-1])
+
+
+_fast_dims_cache = {}
+
+
+def _get_fast_ew_dims(size):
+    """2-D view of a flat contiguous tensor (nervanagpu/float_ew.py:1037-1055);
+    kept for callers that size their launches with it (compensated_sum)."""
+    hit = _fast_dims_cache.get(size)
+    if hit:
+        return hit
+    ew_size = 256
+    while ew_size > 0:
+        if size % ew_size == 0:
+            break
+        ew_size -= 32
+    if ew_size == 0:
+        ew_size = 255
+        while ew_size > 0:
+            if size % ew_size == 0:
+                break
+            ew_size -= 1
+    shape = (size // ew_size, ew_size)
+    res = (shape, _contiguous_strides(shape))
+    _fast_dims_cache[size] = res
+    return res
+
+
+# ---------------------------------------------------------------------------
+# expression tree
+# ---------------------------------------------------------------------------
+
+class _Node(object):
+    """kind: 'tensor' | 'const' | 'op' | 'red'.  key: structural identity used
+    to merge repeated sub-expressions (and in particular repeated reductions)."""
+    __slots__ = ("kind", "name", "args", "arg_id", "key", "level", "scalar", "extra", "op_id")
+
+    def __init__(self, kind, name=None, args=(), arg_id=None, extra=None, op_id=None):
+        self.kind, self.name, self.args, self.arg_id = kind, name, tuple(args), arg_id
+        self.extra, self.op_id = extra, op_id
+        if kind == "tensor":
+            self.key = ("t", arg_id)
+            self.level, self.scalar = 0, False
+        elif kind == "const":
+            self.key = ("c", arg_id)
+            self.level, self.scalar = 0, True
+        elif kind == "red":
+            self.key = ("r", name, args[0].key)
+            self.level, self.scalar = args[0].level + 1, True
+        else:
+            if name in ("rand", "onehot"):
+                self.key = ("o", name, op_id)
+                self.level, self.scalar = 0, False
+            else:
+                self.key = ("o", name) + tuple(a.key for a in args)
+                self.level = max([a.level for a in args] + [0])
+                self.scalar = all(a.scalar for a in args)
+
+
+def _build_tree(type_args):
+    """postfix description -> tree; returns (out_spec, root expression, assign spec)"""
+    stack = []
+    for arg in type_args:
+        kind = arg[0]
+        if kind == "tensor":
+            stack.append(_Node("tensor", arg_id=arg[1]))
+        elif kind == "const":
+            stack.append(_Node("const", arg_id=arg[1]))
+        elif kind == "assign":
+            value = stack.pop()
+            out = stack.pop()
+            assert not stack, "malformed expression stack"
+            return out, value, arg
+        elif kind in _reduction_ops:
+            stack.append(_Node("red", kind, [stack.pop()], op_id=arg[1]))
+        else:
+            nops = _float_ops[kind][0]
+            operands = [stack.pop() for _ in range(nops)][::-1]
+            stack.append(_Node("op", kind, operands, extra=arg[2:], op_id=arg[1]))
+    raise ValueError("expression does not end in an assignment")
+
+
+def _collect_reductions(node, found):
+    for a in node.args:
+        _collect_reductions(a, found)
+    if node.kind == "red" and node.key not in found:
+        found[node.key] = node
+    return found
+
+
+class _Emitter(object):
+    """Turns a tree into HIP source for one kernel specialisation."""
+
+    def __init__(self, spec):
+        self.spec = spec
+        self.lines = []
+        self.names = {}          # key -> variable holding a row-scalar value
+        self.counter = 0
+
+    def fresh(self, prefix="r"):
+        self.counter += 1
+        return "%s%d" % (prefix, self.counter)
+
+    # -- operand access ------------------------------------------------------
+    def load_expr(self, tid, v):
+        """float value of element v of the current vector of tensor tid"""
+        return "x%d_%s[%s]" % (tid, self.cur_item, v)
+
+    def emit_scalar(self, node, out):
+        """value of a row-scalar node, emitted once at workgroup scope"""
+        if node.key in self.names:
+            return self.names[node.key]
+        if node.kind == "const":
+            name = "c%d" % node.arg_id
+        elif node.kind == "red":
+            raise AssertionError("reduction used before its stage")
+        else:
+            ops = [self.emit_scalar(a, out) for a in node.args]
+            name = self.fresh("s")
+            out.append("    const float %s = %s;" % (name, _float_ops[node.name][1].format(*ops)))
+        self.names[node.key] = name
+        return name
+
+    def emit_elem(self, node, out, local, item, v):
+        """value of a node for element (item, v) of the row, emitted in a loop body"""
+        if node.scalar:
+            return self.names[node.key] if node.key in self.names else self._late_scalar(node)
+        if node.key in local:
+            return local[node.key]
+        if node.kind == "tensor":
+            name = self.spec.tensor_value(node.arg_id, item, v)
+        elif node.name == "rand":
+            name = self.fresh("e")
+            out.append("            const float %s = ng_frand(rng_seed, rng_stream + %du, rng_idx + %s);"
+                       % (name, 0x1000193 * (node.op_id + 1) & 0xFFFFFFFF, v))
+        elif node.name == "onehot":
+            name = self.fresh("e")
+            hot_axis, slot = node.extra
+            test = "(col + %s)" % v if hot_axis == 1 else "row"
+            idx = "oh%d_v" % slot if hot_axis == 0 else "oh%d_row" % slot
+            if hot_axis == 0:
+                out.append("            const float %s = (oh%d[col + %s] == %s) ? 1.0f : 0.0f;" % (name, slot, v, "row"))
+            else:
+                out.append("            const float %s = (%s == %s) ? 1.0f : 0.0f;" % (name, idx, test))
+        else:
+            ops = [self.emit_elem(a, out, local, item, v) for a in node.args]
+            name = self.fresh("e")
+            out.append("            const float %s = %s;" % (name, _float_ops[node.name][1].format(*ops)))
+        local[node.key] = name
+        return name
+
+    def _late_scalar(self, node):
+        raise AssertionError("row-scalar %r was not materialised before use" % (node.key,))
+
+    def prepare_scalars(self, node, out, max_level):
+        """emit every row-scalar subtree of `node` whose reductions are done"""
+        if node.scalar:
+            if node.kind == "red":
+                assert node.key in self.names
+                return
+            if node.level <= max_level:
+                self.emit_scalar_tree(node, out)
+            return
+        for a in node.args:
+            self.prepare_scalars(a, out, max_level)
+
+    def emit_scalar_tree(self, node, out):
+        if node.key in self.names:
+            return self.names[node.key]
+        if node.kind == "red":
+            raise AssertionError("reduction not computed yet")
+        return self.emit_scalar(node, out)
+
+
+class KernelSpec(object):
+    """Everything that selects a generated kernel (hashable via .key)."""
+
+    def __init__(self, type_args, tensors, mode, vec, threads, items, n_onehot):
+        # tensors: list of (arg_id, dtype_code, access, take_axis, is_out)
+        #   access: 'vec' contiguous+aligned along the row, 'strided', 'row' (one value per row)
+        self.type_args = tuple(type_args)
+        self.tensors = tuple(tensors)
+        self.mode = mode              # 'flat' | 'row'
+        self.vec = vec
+        self.threads = threads
+        self.items = items            # >0: row cached in registers with this many vectors per lane; 0: streaming
+        self.n_onehot = n_onehot
+        self.key = (self.type_args, self.tensors, mode, vec, threads, items, n_onehot)
+        self._tensor_by_id = dict((t[0], t) for t in tensors)
+
+    def tensor_value(self, arg_id, item, v):
+        t = self._tensor_by_id[arg_id]
+        if t[2] == "row":
+            return "x%d_row" % arg_id
+        return "x%d_%s[%s]" % (arg_id, item, v)
+
+
+def _ctype(code):
+    return _ew_types[code][0]
+
+
+def _gen_load(spec, t, item, base_col, out, indent, bound="n"):
+    """code that fills float x<id>_<item>[VEC] for the vector starting at column base_col"""
+    arg_id, code, access, take_axis, _ = t
+    V = spec.vec
+    ct = _ctype(code)
+    pad = " " * indent
+    if access == "row":
+        return
+    out.append("%sfloat x%d_%s[%d];" % (pad, arg_id, item, V))
+    if access == "vec" and V > 1:
+        out.append("%s{ typedef %s vt_ __attribute__((ext_vector_type(%d)));" % (pad, ct, V))
+        out.append("%s  const vt_ raw_ = *reinterpret_cast<const vt_*>(p%d + (long)(%s));" % (pad, arg_id, base_col))
+        out.append("%s  _Pragma(\"unroll\") for (int v = 0; v < %d; v++) x%d_%s[v] = (float)raw_[v]; }" % (pad, V, arg_id, item))
+    else:
+        if take_axis == 2:
+            idx = "(long)take%d[%s + v]" % (arg_id, base_col)
+        else:
+            idx = "(long)(%s + v) * cs%d" % (base_col, arg_id)
+        out.append("%s_Pragma(\"unroll\") for (int v = 0; v < %d; v++)" % (pad, V))
+        out.append("%s    x%d_%s[v] = (%s + v < %s) ? (float)p%d[%s] : 0.0f;" % (pad, arg_id, item, base_col, bound, arg_id, idx))
+
+
+def _gen_round(code, value, rounding, idx):
+    """expression of storage type for fp32 `value`"""
+    ct, rng = _ew_types[code]
+    if code == "f4":
+        if rounding:
+            return "ng_sr_f32(%s, sr_bits, ng_rand32(rng_seed, rng_stream, %s))" % (value, idx)
+        return value
+    if code == "f2":
+        if rounding:
+            return "__builtin_bit_cast(_Float16, ng_sr_f16(%s, sr_bits, ng_rand32(rng_seed, rng_stream, %s)))" % (value, idx)
+        return "(_Float16)(%s)" % value
+    return "(%s)ng_rint_sat(%s, %rf, %rf)" % (ct, value, rng[0], rng[1])
+
+
+def generate_source(spec, name="ew_kernel"):
+    """HIP source of the kernel described by `spec`.
+    Returns (source, arg_order) where arg_order lists the launch arguments:
+    ('ptr', id) ('rs', id) ('cs', id) ('take', id) ('const', id) ('onehot', slot)
+    ('n',) ('n_out',) ('rows',) ('sr_bits',) ('rng_seed',) ('rng_stream',) ('rng_rm',) ('rng_cm',)"""
+    out_node, root, assign = _build_tree(spec.type_args)
+    rounding = bool(assign[2])
+    reds = list(_collect_reductions(root, {}).values())
+    reds.sort(key=lambda r: r.level)
+    levels = sorted(set(r.level for r in reds))
+    V, T, ITEMS = spec.vec, spec.threads, spec.items
+    flat = spec.mode == "flat"
+    out_t = [t for t in spec.tensors if t[4]][0]
+    in_ts = [t for t in spec.tensors if not t[4]]
+    red_out = root.scalar and not flat   # one value per row: lane 0 stores it
+
+    args, decl = [], []
+    for t in spec.tensors:
+        arg_id, code, access, take_axis, is_out = t
+        const = "" if is_out else "const "
+        decl.append("%s%s* __restrict__ p%d" % (const, _ctype(code), arg_id))
+        args.append(("ptr", arg_id))
+        if not flat:
+            decl.append("int rs%d" % arg_id); args.append(("rs", arg_id))
+            decl.append("int cs%d" % arg_id); args.append(("cs", arg_id))
+        if take_axis:
+            decl.append("const int* __restrict__ take%d" % arg_id); args.append(("take", arg_id))
+    consts = sorted(set(a[1] for a in spec.type_args if a[0] == "const"))
+    for c in consts:
+        decl.append("float c%d" % c); args.append(("const", c))
+    for s in range(spec.n_onehot):
+        decl.append("const int* __restrict__ oh%d" % s); args.append(("onehot", s))
+    decl.append("int n"); args.append(("n",))
+    decl.append("int n_out"); args.append(("n_out",))
+    decl.append("long rows"); args.append(("rows",))
+    decl += ["unsigned sr_bits", "unsigned rng_seed", "unsigned rng_stream", "unsigned rng_rm", "unsigned rng_cm"]
+    args += [("sr_bits",), ("rng_seed",), ("rng_stream",), ("rng_rm",), ("rng_cm",)]
+
+    em = _Emitter(spec)
+    L = []
+    L.append(_lib.common_header_text())
+    L.append("#define THREADS %d" % T)
+    L.append("#define VEC %d" % V)
+    L.append("extern \"C\" __global__ __launch_bounds__(THREADS) void %s(\n    %s)\n{" % (name, ",\n    ".join(decl)))
+    L.append("    const int tid = threadIdx.x;")
+
+    def store_code(item, base_col, vals, indent):
+        pad = " " * indent
+        arg_id, code, access, take_axis, _ = out_t
+        ct = _ctype(code)
+        o = []
+        if access == "vec" and V > 1:
+            o.append("%s{ typedef %s vt_ __attribute__((ext_vector_type(%d))); vt_ o_;" % (pad, ct, V))
+            for v in range(V):
+                o.append("%s  o_[%d] = %s;" % (pad, v, _gen_round(code, vals[v], rounding, "rng_idx + %du" % v if not rng_strided else "rng_idx + %du * rng_cm" % v)))
+            o.append("%s  *reinterpret_cast<vt_*>(p%d + (long)(%s)) = o_; }" % (pad, arg_id, base_col))
+        else:
+            for v in range(V):
+                if take_axis == 2:
+                    idx = "(long)take%d[%s + %d]" % (arg_id, base_col, v)
+                else:
+                    idx = "(long)(%s + %d) * cs%d" % (base_col, v, arg_id)
+                rid = "rng_idx + %du" % v if not rng_strided else "rng_idx + %du * rng_cm" % v
+                o.append("%sif (%s + %d < n_out) p%d[%s] = %s;" % (pad, base_col, v, arg_id, idx, _gen_round(code, vals[v], rounding, rid)))
+        return o
+
+    uses_rand = any(a[0] == "rand" for a in spec.type_args)
+    need_idx = rounding or uses_rand
+
+    if flat:
+        rng_strided = False
+        # one flat grid-stride loop over vectors of VEC consecutive elements
+        L.append("    const long nvec = rows;   // number of VEC-wide vectors")
+        L.append("    for (long g = (long)blockIdx.x * THREADS + tid; g < nvec; g += (long)gridDim.x * THREADS) {")
+        L.append("        const long col = g * VEC;")
+        L.append("        const unsigned rng_idx = (unsigned)col;")
+        body = []
+        for t in in_ts:
+            arg_id, code, access, _, _ = t
+            ct = _ctype(code)
+            body.append("        float x%d_i[%d];" % (arg_id, V))
+            if V > 1:
+                body.append("        { typedef %s vt_ __attribute__((ext_vector_type(%d)));" % (ct, V))
+                body.append("          const vt_ raw_ = *reinterpret_cast<const vt_*>(p%d + col);" % arg_id)
+                body.append("          _Pragma(\"unroll\") for (int v = 0; v < %d; v++) x%d_i[v] = (float)raw_[v]; }" % (V, arg_id))
+            else:
+                body.append("        x%d_i[0] = (float)p%d[col];" % (arg_id, arg_id))
+        for c in consts:
+            em.names[("c", c)] = "c%d" % c
+        vals = []
+        for v in range(V):
+            local = {}
+            blk = []
+            em.prepare_scalars(root, blk, 0)
+            vals.append(em.emit_elem(root, blk, local, "i", str(v)) if not root.scalar else em.emit_scalar_tree(root, blk))
+            body += ["    " + b[4:] if b.startswith("            ") else b for b in blk]
+        L += body
+        arg_id, code, _, _, _ = out_t
+        ct = _ctype(code)
+        if V > 1:
+            L.append("        { typedef %s vt_ __attribute__((ext_vector_type(%d))); vt_ o_;" % (ct, V))
+            for v in range(V):
+                L.append("          o_[%d] = %s;" % (v, _gen_round(code, vals[v], rounding, "rng_idx + %du" % v)))
+            L.append("          *reinterpret_cast<vt_*>(p%d + col) = o_; }" % arg_id)
+        else:
+            L.append("        p%d[col] = %s;" % (arg_id, _gen_round(code, vals[0], rounding, "rng_idx")))
+        L.append("    }")
+        L.append("}")
+        return "\n".join(L), args
+
+    # ---------------- row mode ----------------
+    rng_strided = True
+    L.append("    const int lane = tid & 63, wave = tid >> 6;")
+    L.append("    const long row = blockIdx.x;")
+    L.append("    if (row >= rows) return;")
+    L.append("    __shared__ float red_f[THREADS / 64 + 1];")
+    L.append("    __shared__ int red_i[THREADS / 64 + 1];")
+    L.append("    (void)lane; (void)wave; (void)red_f; (void)red_i;")
+    for t in spec.tensors:
+        arg_id, code, access, take_axis, is_out = t
+        if take_axis == 1:
+            L.append("    p%d += (long)take%d[row] * rs%d;" % (arg_id, arg_id, arg_id))
+        else:
+            L.append("    p%d += row * rs%d;" % (arg_id, arg_id))
+        if access == "row" and not is_out:
+            L.append("    const float x%d_row = (float)p%d[0];" % (arg_id, arg_id))
+    for s in range(spec.n_onehot):
+        L.append("    const int oh%d_row = oh%d[row]; (void)oh%d_row;" % (s, s, s))
+    for c in consts:
+        em.names[("c", c)] = "c%d" % c
+
+    loaded = set()
+
+    def loop_open(bound):
+        if ITEMS:
+            return ["    _Pragma(\"unroll\") for (int it = 0; it < %d; it++) {" % ITEMS,
+                    "        const int col = (it * THREADS + tid) * VEC;",
+                    "        if (col < %s) {" % bound]
+        return ["    for (int col = tid * VEC; col < %s; col += THREADS * VEC) {" % bound, "        {"]
+
+    def needed_tensors(node, acc):
+        if node.kind == "tensor":
+            acc.add(node.arg_id)
+        if node.kind != "red":
+            for a in node.args:
+                needed_tensors(a, acc)
+        return acc
+
+    cached = bool(ITEMS)
+    if cached:
+        # read every streamed operand once into registers
+        for t in in_ts:
+            if t[2] == "row":
+                continue
+            L.append("    float x%d_c[%d][%d];" % (t[0], ITEMS, V))
+        L += loop_open("n")
+        for t in in_ts:
+            if t[2] == "row":
+                continue
+            tmp = []
+            _gen_load(spec, t, "l", "col", tmp, 12)
+            L += tmp
+            L.append("            _Pragma(\"unroll\") for (int v = 0; v < %d; v++) x%d_c[it][v] = x%d_l[v];" % (V, t[0], t[0]))
+        L.append("        }")
+        L.append("    }")
+
+    def tensor_val(arg_id, item, v):
+        t = spec._tensor_by_id[arg_id]
+        if t[2] == "row":
+            return "x%d_row" % arg_id
+        if cached:
+            return "x%d_c[it][%s]" % (arg_id, v)
+        return "x%d_l[%s]" % (arg_id, v)
+    spec.tensor_value = tensor_val
+
+    def block_reduce(kind, var, ivar=None):
+        o = []
+        comb = {"sum": "{0} += {1};", "max": "{0} = fmaxf({0}, {1});", "min": "{0} = fminf({0}, {1});"}
+        if kind in comb:
+            o.append("    _Pragma(\"unroll\") for (int off = 32; off > 0; off >>= 1) { const float o_ = __shfl_xor(%s, off, 64); %s }"
+                     % (var, comb[kind].format(var, "o_")))
+            if T > 64:
+                o.append("    __syncthreads(); if (lane == 0) red_f[wave] = %s; __syncthreads();" % var)
+                o.append("    %s = red_f[0];" % var)
+                o.append("    _Pragma(\"unroll\") for (int w = 1; w < THREADS / 64; w++) { const float o_ = red_f[w]; %s }"
+                         % comb[kind].format(var, "o_"))
+        else:
+            better = ">" if kind == "argmax" else "<"
+            merge = ("if (o_ %s %s || (o_ == %s && oi_ >= 0 && (oi_ < %s || %s < 0))) { %s = o_; %s = oi_; }"
+                     % (better, var, var, ivar, ivar, var, ivar))
+            o.append("    _Pragma(\"unroll\") for (int off = 32; off > 0; off >>= 1) { const float o_ = __shfl_xor(%s, off, 64); const int oi_ = __shfl_xor(%s, off, 64); %s }"
+                     % (var, ivar, merge))
+            if T > 64:
+                o.append("    __syncthreads(); if (lane == 0) { red_f[wave] = %s; red_i[wave] = %s; } __syncthreads();" % (var, ivar))
+                o.append("    %s = red_f[0]; %s = red_i[0];" % (var, ivar))
+                o.append("    _Pragma(\"unroll\") for (int w = 1; w < THREADS / 64; w++) { const float o_ = red_f[w]; const int oi_ = red_i[w]; %s }" % merge)
+        return o
+
+    for lvl in levels:
+        stage = [r for r in reds if r.level == lvl]
+        pre = []
+        for r in stage:
+            em.prepare_scalars(r.args[0], pre, lvl - 1)
+        L += pre
+        for r in stage:
+            var = em.fresh("red")
+            r.extra = var
+            if r.name == "sum":
+                L.append("    float %s = 0.0f;" % var)
+            elif r.name == "max":
+                L.append("    float %s = -3.402823466e+38f;" % var)
+            elif r.name == "min":
+                L.append("    float %s = 3.402823466e+38f;" % var)
+            elif r.name == "argmax":
+                L.append("    float %s = -3.402823466e+38f; int %s_i = -1;" % (var, var))
+            else:
+                L.append("    float %s = 3.402823466e+38f; int %s_i = -1;" % (var, var))
+        L += loop_open("n")
+        if not cached:
+            need = set()
+            for r in stage:
+                needed_tensors(r.args[0], need)
+            for t in in_ts:
+                if t[0] in need and t[2] != "row":
+                    tmp = []
+                    _gen_load(spec, t, "l", "col", tmp, 12)
+                    L += tmp
+        if need_idx:
+            L.append("            const unsigned rng_idx = (unsigned)row * rng_rm + (unsigned)col * rng_cm; (void)rng_idx;")
+        for v in range(V):
+            L.append("            if (col + %d < n) {" % v)
+            local, blk = {}, []
+            for r in stage:
+                val = em.emit_elem(r.args[0], blk, local, "it", str(v)) if not r.args[0].scalar \
+                    else em.names[r.args[0].key]
+                var = r.extra
+                if r.name == "sum":
+                    blk.append("            %s += %s;" % (var, val))
+                elif r.name == "max":
+                    blk.append("            %s = fmaxf(%s, %s);" % (var, var, val))
+                elif r.name == "min":
+                    blk.append("            %s = fminf(%s, %s);" % (var, var, val))
+                elif r.name == "argmax":
+                    blk.append("            if (%s > %s) { %s = %s; %s_i = col + %d; }" % (val, var, var, val, var, v))
+                else:
+                    blk.append("            if (%s < %s) { %s = %s; %s_i = col + %d; }" % (val, var, var, val, var, v))
+            L += ["    " + b for b in blk]
+            L.append("            }")
+        L.append("        }")
+        L.append("    }")
+        for r in stage:
+            var = r.extra
+            if r.name in ("argmax", "argmin"):
+                L += block_reduce(r.name, var, var + "_i")
+                res = em.fresh("s")
+                L.append("    const float %s = (float)%s_i;" % (res, var))
+                em.names[r.key] = res
+            else:
+                L += block_reduce(r.name, var)
+                em.names[r.key] = var
+
+    # final stage
+    pre = []
+    em.prepare_scalars(root, pre, max(levels + [0]))
+    L += pre
+    if red_out:
+        val = em.emit_scalar_tree(root, L)
+        arg_id, code = out_t[0], out_t[1]
+        L.append("    if (tid == 0) {")
+        L.append("        const unsigned rng_idx = (unsigned)row * rng_rm; (void)rng_idx;")
+        L.append("        p%d[0] = %s;" % (arg_id, _gen_round(code, val, rounding, "rng_idx")))
+        L.append("    }")
+    else:
+        L += loop_open("n_out")
+        if not cached:
+            need = needed_tensors(root, set())
+            for t in in_ts:
+                if t[0] in need and t[2] != "row":
+                    tmp = []
+                    _gen_load(spec, t, "l", "col", tmp, 12, "n_out")
+                    L += tmp
+        L.append("            const unsigned rng_idx = (unsigned)row * rng_rm + (unsigned)col * rng_cm; (void)rng_idx;")
+        vals = []
+        for v in range(V):
+            local, blk = {}, []
+            if root.scalar:
+                vals.append(em.emit_scalar_tree(root, blk))
+            else:
+                vals.append(em.emit_elem(root, blk, local, "it", str(v)))
+            L += blk
+        L += store_code("it", "col", vals, 12)
+        L.append("        }")
+        L.append("    }")
+    L.append("}")
+    return "\n".join(L), args
+
+
+# ---------------------------------------------------------------------------
+# host side: marshal a postfix stack into a kernel spec + launch arguments
+# ---------------------------------------------------------------------------
+
+_kernel_cache = {}
+
+
+def _get_kernel(spec):
+    hit = _kernel_cache.get(spec.key)
+    if hit is None:
+        name = "ew_%d" % len(_kernel_cache)
+        source, arg_order = generate_source(spec, name)
+        module = _lib.Module(source, name)
+        hit = (module.get_function(name), arg_order, source)
+        _kernel_cache[spec.key] = hit
+    return hit
+
+
+def _pow2_at_least(x):
+    p = 1
+    while p < x:
+        p *= 2
+    return p
+
+
+class _Plan(object):
+    """Result of analysing one expression stack: kernel spec + argument values."""
+    pass
+
+
+def analyse(args):
+    """Shape/stride/broadcast analysis of a postfix stack
+    (follows nervanagpu/float_ew.py:1058-1286).  Pure host logic: needs no GPU,
+    tensors only need .shape/.strides/.dtype/.size/.is_trans/.take_array/
+    .is_contiguous/.gpudata/.rounding."""
+    from .nervanagpu import GPUTensor
+
+    out = None
+    reduction = False
+    broadcast = transpose = takeop = False
+    contiguous = True
+    argminmax = False
+    axis = 1
+    for arg in args:
+        if type(arg) is dict:
+            op_name = arg["op"]
+            if op_name in _reduction_ops:
+                if op_name[0:3] == "arg":
+                    argminmax = True
+                if arg.get("axis", None) not in (0, 1):
+                    raise ValueError("Only reduction along an axis currently supported")
+                if reduction is True:
+                    if arg["axis"] != axis:
+                        raise ValueError("Reduction only allowed along one axis per kernel.")
+                else:
+                    reduction = True
+                    axis = arg["axis"]
+            elif op_name == "onehot":
+                takeop = True
+        elif isinstance(arg, GPUTensor):
+            if len(arg.shape) < 2 or (len(arg.shape) == 2 and (arg.shape[0] == 1 or arg.shape[1] == 1)):
+                broadcast = True
+            elif arg.is_trans:
+                transpose = True
+            elif arg.take_array:
+                takeop = True
+            elif not arg.is_contiguous:
+                contiguous = False
+
+    complex_op = broadcast or reduction or transpose or takeop or not contiguous
+    stride_order = 1 if axis == 1 else -1
+
+    plan = _Plan()
+    type_args, tensors_info = [], []
+    array_ids, const_ids = {}, {}
+    arg_cnt = op_cnt = 0
+    shape_stack = []
+    values = {}
+    onehots = []
+    max_shape = [1, 1]
+    flat_size = None
+    red_depth = 0
+
+    for arg in args:
+        if isinstance(arg, GPUTensor):
+            if complex_op:
+                if len(arg.shape) == 2:
+                    shape = tuple(arg.shape)
+                    strides = list(arg.strides[::stride_order])
+                elif len(arg.shape) < 2:
+                    # 0-d / 1-d operands broadcast as a row vector
+                    n = arg.size
+                    shape = (1, n)
+                    strides = [0, arg.strides[0] if arg.strides else 0][::stride_order]
+                else:
+                    raise ValueError("Operations that are not simple elementwise are only currently supported in 2 dimensions.")
+            else:
+                shape = (1, arg.size)
+                strides = [0, 1]
+                if flat_size is None:
+                    flat_size = arg.size
+                elif flat_size != arg.size:
+                    raise TypeError("Input shape:%s not compatible" % (arg.shape,))
+
+            key = id(arg)
+            first_out = out is None
+            if first_out:
+                out = arg
+                indx = arg_cnt
+                arg_cnt += 1
+                new = True
+            elif key in array_ids:
+                indx = array_ids[key]
+                new = False
+            else:
+                indx = array_ids[key] = arg_cnt
+                arg_cnt += 1
+                new = True
+
+            if new:
+                if complex_op:
+                    if shape[0] == 1:
+                        strides[1 - axis] = 0
+                    if shape[1] == 1:
+                        strides[axis] = 0
+                take_axis = 0
+                take_ptr = None
+                if arg.take_array:
+                    take_axis = (2 - arg.take_array[1]) if axis != 1 else (arg.take_array[1] + 1)
+                    take_ptr = arg.take_array[0].gpudata
+                values[indx] = dict(ptr=int(arg.gpudata) if arg.gpudata is not None else 0,
+                                    rs=int(strides[0]), cs=int(strides[1]), take=take_ptr,
+                                    dtype=arg.dtype.str[1:], take_axis=take_axis, is_out=first_out,
+                                    itemsize=arg.dtype.itemsize)
+            type_args.append(("tensor", indx))
+            shape_stack.append(shape)
+
+        elif type(arg) in (int, float) or isinstance(arg, (np.integer, np.floating)):
+            val = float(arg)
+            if val in const_ids:
+                indx = const_ids[val]
+            else:
+                indx = const_ids[val] = arg_cnt
+                arg_cnt += 1
+                values[indx] = dict(const=val)
+            type_args.append(("const", indx))
+            shape_stack.append((1, 1))
+
+        elif type(arg) is dict:
+            op_name = arg["op"]
+            if op_name in _float_ops:
+                max_shape = [1, 1]
+                for _ in range(_float_ops[op_name][0]):
+                    shape = shape_stack.pop()
+                    for i in range(2):
+                        if shape[i] != max_shape[i]:
+                            if shape[i] == 1 or max_shape[i] == 1:
+                                max_shape[i] = max(max_shape[i], shape[i])
+                            else:
+                                raise TypeError("Input shape:%s not compatible" % (shape,))
+                if op_name == "assign":
+                    rounding = out.rounding
+                    if rounding:
+                        if rounding is True:
+                            rounding = 10
+                        elif out.dtype.type is np.float32:
+                            rounding = min(rounding, 15)
+                        elif out.dtype.type is np.float16:
+                            rounding = min(rounding, 10)
+                        rounding = max(int(rounding), 1)
+                        if out.dtype.kind != "f":
+                            rounding = 0   # integer outputs always round to nearest
+                    plan.rounding = int(rounding or 0)
+                    type_args.append(("assign", op_cnt, plan.rounding > 0))
+                elif op_name == "onehot":
+                    hot_axis = arg["axis"] if axis else 1 - arg["axis"]
+                    type_args.append(("onehot", op_cnt, hot_axis, len(onehots)))
+                    onehots.append(arg["idx"].gpudata)
+                    shape_stack.append(tuple(max_shape) if len(shape_stack) else (1, 1))
+                else:
+                    type_args.append((op_name, op_cnt))
+                    shape_stack.append(tuple(max_shape))
+            elif op_name in _reduction_ops:
+                shape = list(shape_stack.pop())
+                type_args.append((op_name, op_cnt))
+                red_depth = max(red_depth, shape[axis])
+                shape[axis] = 1
+                shape_stack.append(tuple(shape))
+            else:
+                raise TypeError("%s is not a valid operation" % op_name)
+            op_cnt += 1
+        else:
+            raise TypeError("args must be instance of GPUTensor, int, float, or dict (for operators)")
+
+    if out is None:
+        raise TypeError("expression has no output tensor")
+
+    plan.out = out
+    plan.axis = axis
+    plan.values = values
+    plan.onehots = onehots
+    plan.type_args = type_args
+
+    if not complex_op:
+        size = out.size
+        plan.mode = "flat"
+        # output shape is the broadcast target: assigning a constant is allowed
+        ptr_or = 0
+        for v in values.values():
+            if "ptr" in v:
+                ptr_or |= v["ptr"]
+        vec = 1
+        for cand in (8, 4, 2):
+            ok = size % cand == 0
+            for v in values.values():
+                if "ptr" in v and (v["ptr"] % min(cand * v["itemsize"], 16)) != 0:
+                    ok = False
+            if ok:
+                vec = cand
+                break
+        plan.vec = vec
+        plan.n = plan.n_out = size
+        plan.rows = size // vec
+        plan.threads = 256
+        plan.items = 0
+        plan.grid = max(1, min((plan.rows + 255) // 256, 8192))
+        plan.rng_rm, plan.rng_cm = 0, 1
+        tensors = [(i, v["dtype"], "vec", 0, v["is_out"]) for i, v in sorted(values.items()) if "ptr" in v]
+    else:
+        # the output may be a broadcast target of the expression, never smaller
+        out_shape = tuple(out.shape) if len(out.shape) == 2 else (1, out.size)
+        for i in range(2):
+            if max_shape[i] not in (1, out_shape[i]) and out_shape[i] != 1:
+                raise TypeError("Input shape:%s not compatible" % (tuple(max_shape),))
+        full = [max(max_shape[i], out_shape[i]) for i in range(2)]
+        n_out = full[axis]
+        n = red_depth if reduction else n_out
+        rows = full[1 - axis]
+        plan.mode = "row"
+        plan.n, plan.n_out, plan.rows = n, n_out, rows
+        # logical flat index of (row, col) in the output tensor for the random stream
+        ncols_out = out_shape[1]
+        if axis == 1:
+            plan.rng_rm, plan.rng_cm = ncols_out, 1
+        else:
+            plan.rng_rm, plan.rng_cm = 1, ncols_out
+        vec = 1
+        for cand in (8, 4, 2):
+            ok = n % cand == 0 and (n_out % cand == 0 or n_out == 1)
+            for v in values.values():
+                if "ptr" not in v:
+                    continue
+                if v["take_axis"]:
+                    continue
+                if v["cs"] == 1:
+                    width = min(cand * v["itemsize"], 16)
+                    if v["ptr"] % width or (v["rs"] * v["itemsize"]) % width:
+                        ok = False
+            if ok:
+                vec = cand
+                break
+        if not any(("ptr" in v and v["cs"] == 1 and not v["take_axis"]) for v in values.values()):
+            vec = 1
+        plan.vec = vec
+        nvec = (max(n, n_out) + vec - 1) // vec
+        threads = min(MAX_THREADS, max(64, _pow2_at_least((nvec + 1) // 2)))
+        if not reduction:
+            threads = min(threads, 256)
+        items = (nvec + threads - 1) // threads
+        # keep the row in registers only when every loop walks the same extent
+        if items * vec > MAX_CACHED_PER_LANE or not reduction or n_out not in (1, n):
+            items = 0
+        plan.threads, plan.items = threads, items
+        plan.grid = rows
+        tensors = []
+        for i, v in sorted(values.items()):
+            if "ptr" not in v:
+                continue
+            if v["take_axis"]:
+                access = "strided"
+            elif v["cs"] == 0 and not v["is_out"]:
+                access = "row"
+            elif v["cs"] == 1 and vec > 1:
+                access = "vec"
+            else:
+                access = "strided"
+            tensors.append((i, v["dtype"], access, v["take_axis"], v["is_out"]))
+
+    plan.spec = KernelSpec(type_args, tensors, plan.mode, plan.vec, plan.threads, plan.items, len(onehots))
+    return plan
+
+
+def call_compound_kernel(backend, *args):
+    """Execute a postfix expression stack ending in {"op": "assign"}:
+        C += 2.5 * A * B + 1  ==  (C, 2.5, A, mul, B, mul, 1, add, C, add, assign)
+    `backend` supplies the stream and the random stream (seed, launch counter).
+    Returns the output tensor (nervanagpu/float_ew.py:1058-1322)."""
+    plan = analyse(args)
+    out = plan.out
+    if plan.rows == 0 or plan.n == 0:
+        return out
+    func, arg_order, _ = _get_kernel(plan.spec)
+
+    rounding = plan.rounding
+    uses_rng = rounding or any(a[0] == "rand" for a in plan.type_args)
+    seed, stream_id = backend._next_rng_stream() if uses_rng else (0, 0)
+
+    cargs = []
+    for a in arg_order:
+        kind = a[0]
+        if kind == "ptr":
+            cargs.append(c_void_p(plan.values[a[1]]["ptr"]))
+        elif kind == "rs":
+            cargs.append(c_int(plan.values[a[1]]["rs"]))
+        elif kind == "cs":
+            cargs.append(c_int(plan.values[a[1]]["cs"]))
+        elif kind == "take":
+            cargs.append(c_void_p(int(plan.values[a[1]]["take"])))
+        elif kind == "const":
+            cargs.append(c_float(plan.values[a[1]]["const"]))
+        elif kind == "onehot":
+            cargs.append(c_void_p(int(plan.onehots[a[1]])))
+        elif kind == "n":
+            cargs.append(c_int(plan.n))
+        elif kind == "n_out":
+            cargs.append(c_int(plan.n_out))
+        elif kind == "rows":
+            cargs.append(ctypes.c_long(plan.rows))
+        elif kind == "sr_bits":
+            cargs.append(c_uint(rounding))
+        elif kind == "rng_seed":
+            cargs.append(c_uint(seed))
+        elif kind == "rng_stream":
+            cargs.append(c_uint(stream_id))
+        elif kind == "rng_rm":
+            cargs.append(c_uint(plan.rng_rm))
+        elif kind == "rng_cm":
+            cargs.append(c_uint(plan.rng_cm))
+
+    repeat = backend.bench if isinstance(backend.bench, int) and backend.bench > 1 else 1
+    if repeat > 1:
+        start, end = backend._get_events()
+        start.record(backend.stream)
+    for _ in range(repeat):
+        func.launch((plan.grid, 1, 1), (plan.threads, 1, 1), backend.stream, cargs)
+    if repeat > 1:
+        end.record(backend.stream)
+        end.synchronize()
+        msecs = end.time_since(start) / repeat
+        print("%7.3f msecs shape(%d,%d) blk,thd(%d,%d) %s" %
+              (msecs, plan.rows, plan.n, plan.grid, plan.threads, func.name))
+    return out

@@ -1,0 +1,245 @@
+"""GEMM parity on the GPU: NervanaGPU.dot / batched_dot through the C ABI
+against the numpy oracle (np.dot check of benchmarks/gemm_test.py:27-70,
+all-ones known answer of benchmarks/gemm_test2.py:40-41 and
+kernels/C_interface/test.cu:27-124)."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import oracle as orc
+from util import acc_atol, assert_fp16_within_ulp, assert_fp32_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _operands(ng, op, m, n, k, dtype, rng, lo=-1.0, hi=1.0):
+    A = rng.uniform(lo, hi, (m, k)).astype(dtype)
+    B = rng.uniform(lo, hi, (k, n)).astype(dtype)
+    devA = ng.array(np.ascontiguousarray(A.T) if op[0] == "t" else A, dtype=dtype)
+    devB = ng.array(np.ascontiguousarray(B.T) if op[1] == "t" else B, dtype=dtype)
+    if op[0] == "t":
+        devA = devA.T
+    if op[1] == "t":
+        devB = devB.T
+    return A, B, devA, devB
+
+
+def _absdot(A, B):
+    return np.abs(A.astype(np.float32)) @ np.abs(B.astype(np.float32))
+
+
+def _check(out, ref, dtype, what, atol=0.0):
+    if dtype == np.float16:
+        assert_fp16_within_ulp(out, ref, 1.0, what, atol)
+    else:
+        assert_fp32_close(out, ref, 1e-5, what)
+
+
+SMALL = (1, 2, 3, 7, 8, 9, 16, 33, 64, 65, 127, 128, 192)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("op", ["nn", "nt", "tn"])
+def test_dot_odd_sizes(ng, dtype, op):
+    # subset of the small/medium lists of benchmarks/gemm_test.py:29-31
+    rng = np.random.default_rng(11)
+    sizes = [(m, n, k) for m in SMALL for n in (1, 9, 65, 128) for k in (1, 8, 72, 127)]
+    sizes += [(778, 64, 787), (785, 794, 192), (1, 786, 64), (257, 255, 129), (1537, 64, 1532)]
+    for (m, n, k) in sizes[::3] + sizes[-5:]:
+        A, B, dA, dB = _operands(ng, op, m, n, k, dtype, rng)
+        C = ng.empty((m, n), dtype=dtype)
+        ng.dot(dA, dB, C)
+        _check(C.get(), orc.ref_dot(A, B), dtype, "%s %s m,n,k=%d,%d,%d" % (np.dtype(dtype), op, m, n, k),
+               acc_atol(_absdot(A, B)))
+
+
+@pytest.mark.parametrize("op", ["nn", "tn"])
+def test_config1_fp32_1024(ng, op):
+    rng = np.random.default_rng(0)
+    A = rng.standard_normal((1024, 1024)).astype(np.float32)
+    B = rng.standard_normal((1024, 1024)).astype(np.float32)
+    dA = ng.array(np.ascontiguousarray(A.T), dtype=np.float32).T if op == "tn" else ng.array(A, dtype=np.float32)
+    dB = ng.array(B, dtype=np.float32)
+    C = ng.empty((1024, 1024), dtype=np.float32)
+    ng.dot(dA, dB, C, relu=False)
+    assert_fp32_close(C.get(), orc.ref_dot(A, B), 1e-5, "cfg1 " + op)
+
+
+@pytest.mark.parametrize("size", [257, 256, 255, 129, 128, 127, 65, 64, 17, 16, 15])
+def test_c_api_known_answers(ng, size):
+    """kernels/C_interface/test.cu: sgemm of ones == size everywhere, hgemm of zeros == 0"""
+    from nervanagpu_amd import _lib
+    lib = _lib.load()
+    ones = ng.ones((257, 257), dtype=np.float32)
+    zeros = ng.zeros((257, 257), dtype=np.float16)
+    outf = ng.empty((size, size), dtype=np.float32)
+    outh = ng.ones((size, size), dtype=np.float16)
+    assert lib.nervana_loadKernels(b"../cubin/")
+    assert lib.nervana_randStateSizeBytes() == 2048 * 32 * 4
+    vp = ctypes.c_void_p
+    for a_t, b_t in ((False, False), (False, True), (True, False)):
+        assert lib.nervana_sgemm(vp(ones.ptr), vp(ones.ptr), vp(outf.ptr), a_t, b_t, size, size, size,
+                                 size, size, size, 1.0, 0.0, None, False, False, None, -1)
+        assert np.all(outf.get() == size)
+        assert lib.nervana_hgemm(vp(zeros.ptr), vp(zeros.ptr), vp(outh.ptr), a_t, b_t, size, size, size,
+                                 size, size, size, 1.0, 0.0, None, False, False, None, -1)
+        assert np.all(outh.get() == 0)
+    # column-major wrapper: C_cm = A_cm . B_cm
+    rng = np.random.default_rng(size)
+    m, n, k = size, max(size // 2, 1), size + 3
+    A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    B = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    dA = ng.array(np.asfortranarray(A).T.copy(), dtype=np.float32)   # column-major bytes of A
+    dB = ng.array(np.asfortranarray(B).T.copy(), dtype=np.float32)
+    dC = ng.empty((n, m), dtype=np.float32)
+    assert lib.nervana_sgemm_colmajor(vp(dA.ptr), vp(dB.ptr), vp(dC.ptr), False, False, m, n, k,
+                                      m, k, m, 1.0, 0.0, None, False, False, None, -1)
+    assert_fp32_close(dC.get().T, orc.ref_dot(A, B), 1e-5, "colmajor")
+
+
+def test_all_ones_fp16_known_answer(ng):
+    # benchmarks/gemm_test2.py:40-41: every element equals k, exactly representable in fp16
+    m, n, k = 384, 256, 2048
+    A = ng.ones((m, k), dtype=np.float16)
+    B = ng.ones((k, n), dtype=np.float16)
+    C = ng.empty((m, n), dtype=np.float16)
+    ng.dot(A, B, C)
+    assert np.all(C.get() == k)
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("op", ["nn", "nt", "tn"])
+def test_alpha_beta_relu_and_strided_views(ng, dtype, op):
+    rng = np.random.default_rng(5)
+    m, n, k = 200, 136, 264
+    A, B, dA, dB = _operands(ng, op, m, n, k, dtype, rng)
+    C0 = rng.uniform(-1, 1, (m, n + 8)).astype(dtype)
+    Cbig = ng.array(C0, dtype=dtype)
+    C = Cbig[:, 8:]          # ldc > n, offset pointer
+    for alpha, beta, relu in ((0.5, 0.5, False), (1.0, 0.0, True), (2.0, -1.0, True)):
+        Cbig.set(C0)
+        ng.dot(dA, dB, C, alpha=alpha, beta=beta, relu=relu)
+        got = Cbig.get()
+        ref = orc.ref_dot(A, B, C0[:, 8:], alpha, beta, relu)
+        _check(got[:, 8:], ref, dtype, "alpha/beta/relu %s" % op, acc_atol(abs(alpha) * _absdot(A, B) + 1))
+        assert np.array_equal(got[:, :8], C0[:, :8]), "columns outside the view were modified"
+
+
+FC = [(4096, 9216), (4096, 4096), (1000, 4096)]
+
+
+@pytest.mark.parametrize("MK", FC)
+@pytest.mark.parametrize("op", ["nn", "nt", "tn"])
+@pytest.mark.parametrize("relu", [False, True])
+def test_config2_fc_shapes(ng, MK, op, relu):
+    """fp16 FC-layer shapes with minibatch 128 (op <-> role mapping of benchmarks/cublas.py:68-71)"""
+    M, K = MK
+    N = 128
+    rng = np.random.default_rng(1)
+    if op == "nn":
+        m, n, k = M, N, K
+    elif op == "tn":
+        m, n, k = K, N, M
+    else:
+        m, n, k = M, K, N
+    A, B, dA, dB = _operands(ng, op, m, n, k, np.float16, rng)
+    C = ng.empty((m, n), dtype=np.float16)
+    ng.dot(dA, dB, C, relu=relu)
+    assert_fp16_within_ulp(C.get(), orc.ref_dot(A, B, relu=relu), 1.0, "fc %s %s" % (MK, op),
+                           acc_atol(_absdot(A, B)))
+
+
+def test_config2_square_and_batched(ng):
+    rng = np.random.default_rng(1)
+    A, B, dA, dB = _operands(ng, "nn", 4096, 4096, 4096, np.float16, rng)
+    C = ng.empty((4096, 4096), dtype=np.float16)
+    ng.dot(dA, dB, C)
+    assert_fp16_within_ulp(C.get(), orc.ref_dot(A, B), 1.0, "4096^3", acc_atol(_absdot(A, B)))
+    # linearity: dot(A, 2B) == 2 dot(A, B) exactly (power-of-two scaling)
+    dB2 = ng.array((B * np.float16(2)).astype(np.float16), dtype=np.float16)
+    C2 = ng.empty((4096, 4096), dtype=np.float16)
+    ng.dot(dA, dB2, C2)
+    got, got2 = C.get().astype(np.float32), C2.get().astype(np.float32)
+    fin = (np.abs(got2) < 60000) & (np.abs(got) > 2.0 ** -13)   # fp16 normal range only
+    assert np.array_equal(got[fin] * 2, got2[fin])
+
+    Ab = rng.uniform(-1, 1, (32, 512, 512)).astype(np.float16)
+    Bb = rng.uniform(-1, 1, (32, 512, 512)).astype(np.float16)
+    dAb, dBb = ng.array(Ab, dtype=np.float16), ng.array(Bb, dtype=np.float16)
+    Cb = ng.empty((32, 512, 512), dtype=np.float16)
+    ng.batched_dot(dAb, dBb, Cb)
+    assert_fp16_within_ulp(Cb.get(), orc.ref_batched_dot(Ab, Bb), 1.0, "batched 32x512^3", acc_atol(512 * 0.3))
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_batched_dot_forms(ng, dtype):
+    """fprop / bprop / update forms of benchmarks/batched_dot_test.py:41-74"""
+    rng = np.random.default_rng(9)
+    X, nOut, nIn, N = 5, 96, 72, 32
+    W = rng.uniform(-1, 1, (nOut, nIn)).astype(dtype)
+    I = rng.uniform(-1, 1, (X, nIn, N)).astype(dtype)
+    E = rng.uniform(-1, 1, (X, nOut, N)).astype(dtype)
+    dW, dI, dE = ng.array(W, dtype=dtype), ng.array(I, dtype=dtype), ng.array(E, dtype=dtype)
+    dO = ng.empty((X, nOut, N), dtype=dtype)
+    dB = ng.empty((X, nIn, N), dtype=dtype)
+    dU = ng.empty((nOut, nIn), dtype=dtype)
+    ng.batched_dot(dW, dI, dO)                 # 2-D A broadcast over the batch
+    ng.batched_dot(dW.T, dE, dB)               # transposed 2-D A
+    ng.batched_dot(dE, dI.T, dU)               # summed over the batch into 2-D C
+    _check(dO.get(), orc.ref_batched_dot(W, I), dtype, "fprop", acc_atol(nIn))
+    _check(dB.get(), orc.ref_batched_dot(W.T, E), dtype, "bprop", acc_atol(nOut))
+    _check(dU.get(), orc.ref_batched_dot(E, np.transpose(I, (0, 2, 1)), out_3d=False), dtype, "update",
+           acc_atol(X * N))
+
+
+def test_stochastic_rounding_bit_exact(ng):
+    """SR output bit-exact against the numpy restatement fed the same stream.
+    Operands are small dyadic rationals so every fp32 sum is exact and the
+    pre-rounding value is known without ambiguity."""
+    from nervanagpu_amd import NervanaGPU
+    ngs = NervanaGPU(stochastic_round=10, seed=1234)
+    rng = np.random.default_rng(3)
+    for op, (m, n, k) in (("nn", (256, 128, 192)), ("tn", (130, 72, 64)), ("nt", (64, 264, 40))):
+        A = (rng.integers(-64, 65, (m, k)) / 1024.0).astype(np.float16)
+        B = (rng.integers(-64, 65, (k, n)) / 64.0).astype(np.float16)
+        dA = ngs.array(np.ascontiguousarray(A.T) if op[0] == "t" else A)
+        dB = ngs.array(np.ascontiguousarray(B.T) if op[1] == "t" else B)
+        dA = dA.T if op[0] == "t" else dA
+        dB = dB.T if op[1] == "t" else dB
+        C = ngs.empty((m, n))
+        assert C.rounding == 10
+        ngs.dot(dA, dB, C, relu=True)
+        stream = ngs.rng_counter
+        pre = orc.ref_dot(A, B, relu=True)                      # exact in fp32
+        assert np.array_equal(pre.astype(np.float64), np.maximum(A.astype(np.float64) @ B.astype(np.float64), 0))
+        r = orc.rand32(1234, stream, np.arange(m * n, dtype=np.uint32)).reshape(m, n)
+        exp = orc.round_stochastic_fp16(pre, 10, r)
+        got = C.get()
+        assert np.array_equal(got.view(np.uint16), exp.view(np.uint16)), op
+        # and it is not plain nearest rounding
+        assert not np.array_equal(got.view(np.uint16), pre.astype(np.float16).view(np.uint16))
+    # fp32 output keeps `bits` mantissa bits
+    ngs32 = NervanaGPU(stochastic_round=7, seed=99)
+    A = rng.uniform(-1, 1, (128, 64)).astype(np.float32)
+    B = rng.uniform(-1, 1, (64, 136)).astype(np.float32)
+    C = ngs32.empty((128, 136), dtype=np.float32)
+    ngs32.dot(ngs32.array(A, dtype=np.float32), ngs32.array(B, dtype=np.float32), C)
+    got = C.get()
+    assert np.all((got.view(np.uint32) & ((1 << 16) - 1)) == 0)
+    ref = orc.ref_dot(A, B)
+    assert np.all(np.abs(got - ref) <= 2.0 ** -7 * np.abs(ref) * 1.01 + 1e-5)   # within one unit at 7 bits
+
+
+def test_error_paths(ng):
+    A = ng.empty((8, 8), dtype=np.float16)
+    B = ng.empty((8, 8), dtype=np.float32)
+    with pytest.raises(AssertionError):
+        ng.dot(A, B, A)
+    with pytest.raises(AssertionError):
+        ng.dot(A.T, A.T, A)        # "tt" is not supported
+    with pytest.raises(AssertionError):
+        ng.dot(A, ng.empty((9, 8), dtype=np.float16), A)
+    Ci = ng.empty((8, 8), dtype=np.int8)
+    with pytest.raises((TypeError, AssertionError)):
+        ng.dot(Ci, Ci, Ci)

@@ -1,0 +1,47 @@
+"""Shared helpers of the parity tests."""
+import numpy as np
+
+
+def fp16_ulp(ref):
+    """size of one fp16 unit in the last place at |ref| (float64 array)"""
+    a = np.abs(np.asarray(ref, dtype=np.float64))
+    a16 = np.minimum(a, 65504.0).astype(np.float16)
+    return np.spacing(a16).astype(np.float64)
+
+
+EPS32 = 2.0 ** -24
+
+
+def acc_atol(absdot):
+    """bound on the fp32 accumulation error of a dot product whose absolute
+    terms sum to `absdot`: it only matters where the result cancels to ~0"""
+    return 4.0 * EPS32 * np.asarray(absdot, dtype=np.float64)
+
+
+def assert_fp16_within_ulp(out, ref32, ulps=1.0, what="", atol=0.0):
+    """fp16 result within `ulps` fp16 units of the fp32-accumulated reference
+    (plus `atol`, the accumulation error of the fp32 value itself)"""
+    out = np.asarray(out)
+    assert out.dtype == np.float16, out.dtype
+    ref = np.asarray(ref32, dtype=np.float64)
+    assert out.shape == ref.shape, (out.shape, ref.shape)
+    o = out.astype(np.float64)
+    fin = np.isfinite(ref) & (np.abs(ref) < 65504.0)
+    err = np.abs(o[fin] - ref[fin])
+    atol = np.broadcast_to(np.asarray(atol, dtype=np.float64), ref.shape)[fin]
+    tol = ulps * fp16_ulp(ref[fin]) * (1.0 + 1e-6) + atol
+    bad = err > tol
+    if bad.any():
+        i = np.argmax(err / tol)
+        raise AssertionError("%s: %d of %d elements off by more than %g fp16 ulp (worst: got %r ref %r)"
+                             % (what, bad.sum(), bad.size, ulps, o[fin][i], ref[fin][i]))
+
+
+def assert_fp32_close(out, ref32, rel=1e-5, what=""):
+    """max|d| / mean|ref| <= rel (metric form of benchmarks/cublas_test.py:169-171)"""
+    out = np.asarray(out, dtype=np.float64)
+    ref = np.asarray(ref32, dtype=np.float64)
+    assert out.shape == ref.shape, (out.shape, ref.shape)
+    scale = max(np.abs(ref).mean(), 1e-30)
+    err = np.abs(out - ref).max() / scale
+    assert err <= rel, "%s: max|d|/mean|ref| = %.3g > %.3g" % (what, err, rel)
