@@ -1,0 +1,236 @@
+"""Convolution fprop / bprop / update parity on the GPU against the numpy
+oracle (per-pixel gather + np.dot of benchmarks/conv_test.py:99-167).
+Full-tensor comparison at reduced shapes; sampled pixels / filter rows plus
+border positions at the configured layer shapes."""
+import numpy as np
+import pytest
+
+import oracle as orc
+from util import acc_atol, assert_fp16_within_ulp, assert_fp32_close
+
+pytestmark = pytest.mark.gpu
+
+# N, C, K, D, H, W, T, R, S, pad(d,h,w), stride(d,h,w)
+SMALL = [
+    (16, 3, 8, 1, 64, 64, 1, 3, 3, (0, 1, 1), (1, 1, 1)),        # benchmarks/conv_test.py:36-42
+    (8, 3, 16, 1, 35, 35, 1, 11, 11, (0, 2, 2), (1, 4, 4)),       # strided, C=3 (AlexNet conv1 style)
+    (16, 64, 72, 1, 13, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (32, 40, 64, 1, 14, 9, 1, 5, 3, (0, 2, 0), (1, 2, 1)),
+    (8, 16, 32, 5, 9, 8, 3, 3, 3, (1, 0, 1), (1, 1, 2)),          # 3-D
+    (64, 8, 8, 1, 7, 7, 1, 1, 1, (0, 0, 0), (1, 1, 1)),           # 1x1
+    (8, 20, 24, 1, 12, 12, 1, 2, 2, (0, 0, 0), (1, 3, 3)),        # stride > filter: unreached input pixels
+]
+
+
+def _layer(ng, dtype, case):
+    N, C, K, D, H, W, T, R, S, pad, strd = case
+    return ng.conv_layer(dtype, N, C, K, D, H, W, T, R, S, pad[0], pad[1], pad[2], strd[0], strd[1], strd[2])
+
+
+def _data(layer, dtype, seed):
+    rng = np.random.default_rng(seed)
+    I = rng.uniform(-1, 1, layer.dimI).astype(dtype)
+    F = rng.uniform(-1, 1, layer.dimF).astype(dtype)
+    E = rng.uniform(-1, 1, layer.dimO).astype(dtype)
+    return I, F, E
+
+
+def _check(out, ref, dtype, what, absacc):
+    if np.dtype(dtype) == np.float16:
+        assert_fp16_within_ulp(out, ref, 1.0, what, acc_atol(absacc))
+    else:
+        assert_fp32_close(out, ref, 1e-5, what)
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("case", SMALL)
+def test_conv_small_full_compare(ng, dtype, case):
+    layer = _layer(ng, dtype, case)
+    I, F, E = _data(layer, dtype, 2)
+    dI, dF, dE = ng.array(I, dtype=dtype), ng.array(F, dtype=dtype), ng.array(E, dtype=dtype)
+    crst = layer.dimF2[0]
+
+    dO = ng.empty(layer.dimO, dtype=dtype)
+    ng.fprop_conv(layer, dI, dF, dO, alpha=1.0)
+    _check(dO.get(), orc.ref_conv_fprop(I, F, layer.padding, layer.strides), dtype, "fprop", crst)
+    ng.fprop_conv(layer, dI, dF, dO, alpha=0.5, relu=True)
+    _check(dO.get(), orc.ref_conv_fprop(I, F, layer.padding, layer.strides, 0.5, True), dtype, "fprop relu", crst)
+
+    dB = ng.empty(layer.dimI, dtype=dtype)
+    dB.fill(7)   # every element must be overwritten
+    ng.bprop_conv(layer, dF, dE, dB, alpha=1.0)
+    krst = layer.K * np.prod(layer.TRS)
+    _check(dB.get(), orc.ref_conv_bprop(F, E, layer.dimI, layer.padding, layer.strides), dtype, "bprop", krst)
+
+    ref_u = orc.ref_conv_update(I, E, layer.dimF, layer.padding, layer.strides)
+    depth = np.prod(layer.MPQ) * layer.N
+    dU = ng.empty(layer.dimF, dtype=np.float32)
+    ng.update_conv(layer, dI, dE, dU, alpha=1.0)
+    assert_fp32_close(dU.get(), ref_u, 1e-5, "update fp32 out")
+    if dtype == np.float16:
+        dUh = ng.empty(layer.dimF, dtype=np.float16)
+        ng.update_conv(layer, dI, dE, dUh, alpha=2.0)
+        assert_fp16_within_ulp(dUh.get(), 2 * ref_u, 1.0, "update fp16 out", acc_atol(2 * depth))
+
+
+def test_conv_uint8_input_bit_exact(ng):
+    """bytes are converted exactly on load: the result must equal the run on the
+    same values stored as fp16, bit for bit (README.md:37)"""
+    case = (16, 3, 16, 1, 31, 31, 1, 5, 5, (0, 2, 2), (1, 2, 2))
+    layer = _layer(ng, np.float16, case)
+    rng = np.random.default_rng(4)
+    I8 = rng.integers(0, 256, layer.dimI).astype(np.uint8)
+    F = (rng.standard_normal(layer.dimF) * 0.01).astype(np.float16)
+    E = rng.uniform(-1, 1, layer.dimO).astype(np.float16)
+    dF, dE = ng.array(F), ng.array(E)
+    dI8 = ng.array(I8, dtype=np.uint8)
+    dIh = ng.array(I8.astype(np.float16))
+    O8, Oh = ng.empty(layer.dimO), ng.empty(layer.dimO)
+    ng.fprop_conv(layer, dI8, dF, O8, relu=True)
+    ng.fprop_conv(layer, dIh, dF, Oh, relu=True)
+    assert np.array_equal(O8.get().view(np.uint16), Oh.get().view(np.uint16))
+    assert_fp16_within_ulp(O8.get(), orc.ref_conv_fprop(I8.astype(np.float32), F, layer.padding, layer.strides, 1.0, True),
+                           1.0, "u8 fprop", acc_atol(255.0 * 75))
+    U8, Uh = ng.empty(layer.dimF, dtype=np.float32), ng.empty(layer.dimF, dtype=np.float32)
+    ng.update_conv(layer, dI8, dE, U8)
+    ng.update_conv(layer, dIh, dE, Uh)
+    assert np.array_equal(U8.get(), Uh.get())
+    # signed bytes
+    Is8 = rng.integers(-128, 128, layer.dimI).astype(np.int8)
+    ng.fprop_conv(layer, ng.array(Is8, dtype=np.int8), dF, O8)
+    ng.fprop_conv(layer, ng.array(Is8.astype(np.float16)), dF, Oh)
+    assert np.array_equal(O8.get().view(np.uint16), Oh.get().view(np.uint16))
+
+
+def test_conv_adjoint_identity_gpu(ng):
+    """<fprop(I,F),E> == <I,bprop(F,E)> == <F,update(I,E)> with fp32 tensors"""
+    case = (16, 24, 40, 1, 17, 15, 1, 3, 5, (0, 1, 2), (1, 2, 1))
+    layer = _layer(ng, np.float32, case)
+    I, F, E = _data(layer, np.float32, 5)
+    dI, dF, dE = (ng.array(x, dtype=np.float32) for x in (I, F, E))
+    dO, dB, dU = (ng.empty(s, dtype=np.float32) for s in (layer.dimO, layer.dimI, layer.dimF))
+    ng.fprop_conv(layer, dI, dF, dO)
+    ng.bprop_conv(layer, dF, dE, dB)
+    ng.update_conv(layer, dI, dE, dU)
+    a = np.vdot(dO.get().astype(np.float64), E)
+    b = np.vdot(I, dB.get().astype(np.float64))
+    c = np.vdot(F, dU.get().astype(np.float64))
+    assert abs(a - b) <= 1e-5 * abs(a) and abs(a - c) <= 1e-5 * abs(a)
+
+
+ALEXNET = [  # C,H,W,K,R,S,stride,pad at N=128 (BASELINE config 3)
+    (3, 224, 224, 64, 11, 11, 4, 2), (64, 27, 27, 192, 5, 5, 1, 2), (192, 13, 13, 384, 3, 3, 1, 1),
+    (384, 13, 13, 256, 3, 3, 1, 1), (256, 13, 13, 256, 3, 3, 1, 1)]
+VGG = [  # C,HW,K at N=64, 3x3 s1 p1 (BASELINE config 4)
+    (3, 224, 64), (64, 224, 64), (64, 112, 128), (128, 112, 128), (128, 56, 256), (256, 56, 256),
+    (256, 28, 512), (512, 28, 512), (512, 14, 512)]
+
+
+def _sampled_layer_check(ng, layer, seed, gen, npix=24, nrows=6, in_dtype=np.float16):
+    rng = np.random.default_rng(seed)
+    I, F, E = gen(rng, layer)
+    dI = ng.array(I, dtype=in_dtype)
+    dF, dE = ng.array(F), ng.array(E)
+    M, P, Q = layer.MPQ
+    D, H, W = layer.DHW
+    crst = layer.dimF2[0]
+    If = I.astype(np.float32)
+    scale_i, scale_f, scale_e = np.abs(If).max(), np.abs(F.astype(np.float32)).max(), np.abs(E.astype(np.float32)).max()
+
+    def sample(dims):
+        pts = [tuple(int(rng.integers(0, d)) for d in dims) for _ in range(npix)]
+        pts += [tuple(0 for _ in dims), tuple(d - 1 for d in dims), (0, 0, dims[2] - 1), (0, dims[1] - 1, 0)]
+        return pts
+
+    dO = ng.empty(layer.dimO)
+    ng.fprop_conv(layer, dI, dF, dO, relu=True)
+    O = dO.get()
+    pix = sample((M, P, Q))
+    ref = orc.ref_conv_fprop_pixels(If, F, pix, layer.padding, layer.strides, 1.0, True)
+    got = np.stack([O[:, m, p, q, :] for (m, p, q) in pix])
+    assert_fp16_within_ulp(got, ref, 1.0, "fprop %s" % layer, acc_atol(crst * scale_i * scale_f))
+    del O
+
+    if in_dtype == np.float16:
+        dB = ng.empty(layer.dimI)
+        ng.bprop_conv(layer, dF, dE, dB)
+        B = dB.get()
+        ipix = sample((D, H, W))
+        refb = orc.ref_conv_bprop_pixels(F, E, layer.dimI, ipix, layer.padding, layer.strides)
+        gotb = np.stack([B[:, z, y, x, :] for (z, y, x) in ipix])
+        assert_fp16_within_ulp(gotb, refb, 1.0, "bprop %s" % layer,
+                               acc_atol(layer.K * np.prod(layer.TRS) * scale_f * scale_e))
+        del B, dB
+
+    dU = ng.empty(layer.dimF, dtype=np.float32)
+    ng.update_conv(layer, dI, dE, dU)
+    U = dU.get().reshape(crst, layer.K)
+    rows = np.unique(np.concatenate([rng.integers(0, crst, nrows), [0, crst - 1]]))
+    refu = orc.ref_conv_update_rows(If, E, layer.dimF, rows, layer.padding, layer.strides)
+    assert_fp32_close(U[rows], refu, 2e-5, "update %s" % layer)
+
+
+def _alexnet_data(rng, layer):
+    I = rng.uniform(0, 1, layer.dimI).astype(np.float16)
+    F = (rng.standard_normal(layer.dimF) * 0.01).astype(np.float16)
+    E = rng.uniform(-1, 1, layer.dimO).astype(np.float16)
+    E *= (rng.uniform(0, 1, layer.dimO) > 0.5)           # relu mask
+    return I, F, E
+
+
+@pytest.mark.parametrize("cfg", ALEXNET)
+def test_config3_alexnet_layers(ng, cfg):
+    C, H, W, K, R, S, strd, pad = cfg
+    layer = ng.conv_layer(np.float16, 128, C, K, 1, H, W, 1, R, S, 0, pad, pad, 1, strd, strd)
+    _sampled_layer_check(ng, layer, 2, _alexnet_data, npix=12 if C * R * S > 2000 else 24)
+
+
+def test_config3_first_layer_uint8(ng):
+    C, H, W, K, R, S, strd, pad = ALEXNET[0]
+    layer = ng.conv_layer(np.float16, 128, C, K, 1, H, W, 1, R, S, 0, pad, pad, 1, strd, strd)
+
+    def gen(rng, layer):
+        I = rng.integers(0, 256, layer.dimI).astype(np.uint8)
+        F = (rng.standard_normal(layer.dimF) * 0.01).astype(np.float16)
+        E = rng.uniform(-1, 1, layer.dimO).astype(np.float16)
+        return I, F, E
+    _sampled_layer_check(ng, layer, 2, gen, in_dtype=np.uint8)
+
+
+@pytest.mark.parametrize("cfg", VGG)
+def test_config4_vgg_layers(ng, cfg):
+    C, HW, K = cfg
+    layer = ng.conv_layer(np.float16, 64, C, K, 1, HW, HW, 1, 3, 3, 0, 1, 1, 1, 1, 1)
+
+    def gen(rng, layer):
+        I = rng.standard_normal(layer.dimI, dtype=np.float32).astype(np.float16)
+        F = (rng.standard_normal(layer.dimF) * np.sqrt(2.0 / (C * 9))).astype(np.float16)
+        E = rng.standard_normal(layer.dimO, dtype=np.float32).astype(np.float16)
+        return I, F, E
+    _sampled_layer_check(ng, layer, 3, gen, npix=10, nrows=3)
+
+
+def test_config5_conv3d(ng):
+    layer = ng.conv_layer(np.float16, 32, 64, 128, 16, 28, 28, 3, 3, 3)
+    assert layer.MPQ == (14, 26, 26)
+
+    def gen(rng, layer):
+        I = rng.uniform(-1, 1, layer.dimI).astype(np.float16)
+        F = (rng.standard_normal(layer.dimF) * 0.05).astype(np.float16)
+        E = rng.uniform(-1, 1, layer.dimO).astype(np.float16)
+        return I, F, E
+    _sampled_layer_check(ng, layer, 4, gen, npix=10, nrows=3)
+
+
+def test_deconv_layer_and_errors(ng):
+    layer = ng.deconv_layer(np.float16, 16, 8, 16, 10, 12, 3, 3, 0, 1, 1, 1, 2, 2)
+    assert layer.MPQ[1:] == (10, 12)
+    with pytest.raises(AssertionError):
+        ng.conv_layer(np.float16, 12, 3, 8, 1, 8, 8, 1, 3, 3)        # N % 8
+    with pytest.raises(AssertionError):
+        ng.conv_layer(np.float16, 16, 3, 6, 1, 8, 8, 1, 3, 3)        # K % 8
+    small = ng.conv_layer(np.float16, 16, 3, 8, 1, 8, 8, 1, 3, 3)
+    with pytest.raises(AssertionError):
+        ng.fprop_conv(small, ng.empty((3, 1, 8, 8, 8)), ng.empty(small.dimF), ng.empty(small.dimO))
+    with pytest.raises(AssertionError):
+        ng.fprop_conv(small, ng.empty(small.dimI), ng.empty(small.dimF, dtype=np.float32), ng.empty(small.dimO))

@@ -1,0 +1,122 @@
+"""Max / average pooling fprop and bprop on the GPU against the numpy oracle
+(gather + np.max/np.argmax/np.mean of benchmarks/pool_test.py:71-146)."""
+import numpy as np
+import pytest
+
+import oracle as orc
+from util import assert_fp16_within_ulp
+
+pytestmark = pytest.mark.gpu
+
+# N, C, D, H, W, J, T, R, S, pad(j,d,h,w), stride(j,d,h,w)
+CASES = [
+    (32, 32, 1, 32, 32, 2, 1, 3, 3, (0, 0, 0, 0), (2, 1, 2, 2)),     # benchmarks/pool_test.py:31-37
+    (64, 16, 1, 16, 16, 1, 1, 2, 2, (0, 0, 0, 0), (1, 1, 2, 2)),     # non-overlapping, tiles exactly
+    (16, 8, 1, 15, 15, 1, 1, 2, 2, (0, 0, 0, 0), (1, 1, 2, 2)),      # ragged edge
+    (8, 12, 1, 13, 13, 1, 1, 3, 3, (0, 0, 1, 1), (1, 1, 2, 2)),      # padded, overlapping
+    (8, 6, 4, 9, 7, 1, 2, 3, 2, (0, 1, 1, 0), (1, 1, 2, 1)),         # 3-D window
+    (24, 9, 1, 6, 6, 3, 1, 1, 1, (0, 0, 0, 0), (3, 1, 1, 1)),        # maxout over feature maps only
+    (12, 5, 1, 9, 9, 1, 1, 3, 3, (0, 0, 0, 0), (1, 1, 4, 4)),        # stride > window: uncovered inputs
+    (4, 4, 1, 8, 8, 1, 1, 3, 3, (0, 0, 0, 0), (1, 1, 1, 1)),         # N not a multiple of 8 (scalar path)
+]
+
+
+def _layer(ng, dtype, op, case):
+    N, C, D, H, W, J, T, R, S, pad, strd = case
+    return ng.pool_layer(dtype, op, N, C, D, H, W, J, T, R, S, pad[0], pad[1], pad[2], pad[3],
+                         strd[0], strd[1], strd[2], strd[3])
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("op", ["max", "avg"])
+@pytest.mark.parametrize("case", CASES)
+def test_pool_full_compare(ng, dtype, op, case):
+    layer = _layer(ng, dtype, op, case)
+    rng = np.random.default_rng(7)
+    I = rng.uniform(0, 1, layer.dimI).astype(np.float16).astype(dtype)
+    E = rng.uniform(-1, 1, layer.dimO).astype(np.float16).astype(dtype)
+    dI, dE = ng.array(I, dtype=dtype), ng.array(E, dtype=dtype)
+    dO = ng.empty(layer.dimO, dtype=dtype)
+    dB = ng.empty(layer.dimI, dtype=dtype)
+    dB.fill(9)
+    ng.fprop_pool(layer, dI, dO)
+    ng.bprop_pool(layer, dI, dE, dB)
+    refO = orc.ref_pool_fprop(I, op, layer.JTRS, layer.padding, layer.strides)
+    refB = orc.ref_pool_bprop(I, E, op, layer.JTRS, layer.padding, layer.strides)
+    if op == "max":
+        assert np.array_equal(dO.get(), refO.astype(dtype))          # max is exact
+    elif dtype == np.float16:
+        assert_fp16_within_ulp(dO.get(), refO, 1.0, "avg fprop", 1e-6)
+    else:
+        np.testing.assert_allclose(dO.get(), refO, rtol=1e-5, atol=1e-6)
+    if dtype == np.float16:
+        assert_fp16_within_ulp(dB.get(), refB, 1.0, "%s bprop" % op, 1e-6)
+    else:
+        np.testing.assert_allclose(dB.get(), refB, rtol=1e-5, atol=1e-6)
+
+
+def test_max_pool_ties_and_out_of_bounds(ng):
+    """first maximum in (j,t,r,s) scan order wins (kernels/sass/hpool_max.sass:264-282)"""
+    layer = ng.pool_layer(np.float16, "max", 8, 4, 1, 6, 6, 1, 1, 3, 3, 0, 0, 1, 1, 1, 1, 1, 1)
+    I = np.ones(layer.dimI, np.float16)          # every window is all ties
+    E = np.full(layer.dimO, 1.0, np.float16)
+    dB = ng.empty(layer.dimI)
+    ng.bprop_pool(layer, ng.array(I), ng.array(E), dB)
+    ref = orc.ref_pool_bprop(I, E, "max", layer.JTRS, layer.padding, layer.strides)
+    assert np.array_equal(dB.get(), ref.astype(np.float16))
+
+
+def test_config4_vgg_pool_shapes(ng):
+    """2x2/2 max pooling at the five block ends of config 4 (reduced in C to bound
+    host time, full in H, W, N); idempotent structure: pooled gradient sums match"""
+    rng = np.random.default_rng(3)
+    for C, HW in ((8, 224), (8, 112), (16, 56), (32, 28), (64, 14)):
+        layer = ng.pool_layer(np.float16, "max", 64, C, 1, HW, HW, 1, 1, 2, 2)
+        I = rng.standard_normal(layer.dimI, dtype=np.float32).astype(np.float16)
+        E = rng.standard_normal(layer.dimO, dtype=np.float32).astype(np.float16)
+        dI, dE = ng.array(I), ng.array(E)
+        dO, dB = ng.empty(layer.dimO), ng.empty(layer.dimI)
+        ng.fprop_pool(layer, dI, dO)
+        ng.bprop_pool(layer, dI, dE, dB)
+        ref = I.astype(np.float32).reshape(C, 1, HW // 2, 2, HW // 2, 2, 64).max(axis=(3, 5))
+        assert np.array_equal(dO.get(), ref.astype(np.float16))
+        B = dB.get().astype(np.float32)
+        # each window passes its error to exactly one element
+        assert np.array_equal(B.reshape(C, 1, HW // 2, 2, HW // 2, 2, 64).sum(axis=(3, 5)), E.astype(np.float32))
+        assert np.count_nonzero(B) <= E.size
+
+
+def test_config5_pool_sampled(ng):
+    """3x3/2 on C=256, 56x56, N=128: sampled windows / pixels vs the oracle"""
+    rng = np.random.default_rng(4)
+    for op in ("max", "avg"):
+        layer = ng.pool_layer(np.float16, op, 128, 256, 1, 56, 56, 1, 1, 3, 3, 0, 0, 0, 0, 1, 1, 2, 2)
+        assert layer.MPQ == (1, 27, 27)
+        I = rng.uniform(0, 1, layer.dimI).astype(np.float16)
+        E = rng.uniform(-1, 1, layer.dimO).astype(np.float16)
+        dI, dE = ng.array(I), ng.array(E)
+        dO, dB = ng.empty(layer.dimO), ng.empty(layer.dimI)
+        ng.fprop_pool(layer, dI, dO)
+        ng.bprop_pool(layer, dI, dE, dB)
+        O = dO.get()
+        wins = [(int(rng.integers(256)), 0, int(rng.integers(27)), int(rng.integers(27))) for _ in range(64)]
+        wins += [(0, 0, 0, 0), (255, 0, 26, 26), (7, 0, 0, 26), (9, 0, 26, 0)]
+        ref = orc.ref_pool_fprop_pixels(I, op, layer.JTRS, wins, layer.padding, layer.strides)
+        got = np.stack([O[w] for w in wins])
+        assert_fp16_within_ulp(got, ref, 1.0 if op == "avg" else 0.0, "%s fprop" % op, 1e-7 if op == "avg" else 0.0)
+        # bprop: compare whole channels against the oracle run on those channels only
+        B = dB.get()
+        for c in (0, 131, 255):
+            refB = orc.ref_pool_bprop(I[c:c + 1], E[c:c + 1], op, layer.JTRS, layer.padding, layer.strides)
+            assert_fp16_within_ulp(B[c:c + 1], refB, 1.0, "%s bprop" % op, 1e-6)
+
+
+def test_pool_errors(ng):
+    layer = ng.pool_layer(np.float16, "l2", 8, 4, 1, 6, 6, 1, 1, 2, 2)
+    with pytest.raises(ValueError):
+        ng.fprop_pool(layer, ng.empty(layer.dimI), ng.empty(layer.dimO))
+    ok = ng.pool_layer(np.float16, "max", 8, 4, 1, 6, 6, 1, 1, 2, 2)
+    with pytest.raises(AssertionError):
+        ng.fprop_pool(ok, ng.empty(layer.dimI), ng.empty((4, 1, 3, 3, 16)))
+    with pytest.raises(AssertionError):
+        ng.bprop_pool(ok, ng.empty(ok.dimI), ng.empty(ok.dimO), ng.empty(ok.dimI, dtype=np.float32))

@@ -42,6 +42,7 @@ def assert_fp32_close(out, ref32, rel=1e-5, what=""):
     out = np.asarray(out, dtype=np.float64)
     ref = np.asarray(ref32, dtype=np.float64)
     assert out.shape == ref.shape, (out.shape, ref.shape)
-    scale = max(np.abs(ref).mean(), 1e-30)
+    nz = ref != 0          # exact zeros (e.g. produced by relu) do not dilute the scale
+    scale = max(np.abs(ref[nz]).mean() if nz.any() else 0.0, 1e-30)
     err = np.abs(out - ref).max() / scale
     assert err <= rel, "%s: max|d|/mean|ref| = %.3g > %.3g" % (what, err, rel)
