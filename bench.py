@@ -1,0 +1,342 @@
+#!/usr/bin/env python3
+"""
+Benchmark of the NervanaGPU compute core on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W        -> ONE JSON line on stdout
+    python bench.py --all [--out FILE]                    -> also a per-case table
+                                                             (GEMM, conv, pool, elementwise)
+
+A "step" is one pass over BASELINE config 2: the fp16 fully-connected GEMM sweep
+with minibatch 128 ((M,K) in {(4096,9216),(4096,4096),(1000,4096)} x nn/nt/tn x
+relu off/on x nearest/stochastic rounding), the square 4096^3 fp16 GEMM and the
+batched 32 x 512^3 GEMM, with every operand already resident in HBM.  `value` is
+the algorithmic flops of one step divided by its wall time.
+
+`roofline` describes the dominant kernel of the step (the 4096^3 fp16 GEMM,
+MFMA bound): algorithmic flops per launch / average launch duration measured
+with HIP events on the launch stream.  `cpu_baseline` times the numpy oracle
+(np.dot, the reference's own CPU check) on a bounded sample of the same step on
+the host cores of the GPU box.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2500.0     # dense fp16 MFMA, MI355X
+PEAK_FP32_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+FC_SHAPES = [(4096, 9216), (4096, 4096), (1000, 4096)]
+MINIBATCH = 128
+
+
+def fc_mnk(op, M, K, N=MINIBATCH):
+    """op <-> fully-connected role (benchmarks/cublas.py:68-71 of the reference)"""
+    if op == "nn":
+        return M, N, K        # fprop  W(M,K) . x(K,N)
+    if op == "tn":
+        return K, N, M        # bprop  W(M,K)^T . d(M,N)
+    return M, K, N            # update d(M,N) . x(K,N)^T
+
+
+class GemmCase(object):
+    def __init__(self, ng, op, m, n, k, relu=False, sr=False, dtype=np.float16, batch=0, seed=1):
+        rng = np.random.default_rng(seed)
+        self.op, self.m, self.n, self.k, self.relu, self.sr, self.batch = op, m, n, k, relu, sr, batch
+        self.dtype = dtype
+        bshape = (batch,) if batch else ()
+        a_shape = bshape + ((k, m) if op[0] == "t" else (m, k))
+        b_shape = bshape + ((n, k) if op[1] == "t" else (k, n))
+        self.hA = rng.uniform(-1, 1, a_shape).astype(dtype)
+        self.hB = rng.uniform(-1, 1, b_shape).astype(dtype)
+        self.A = ng.array(self.hA, dtype=dtype)
+        self.B = ng.array(self.hB, dtype=dtype)
+        self.C = ng.empty(bshape + (m, n), dtype=dtype)
+        self.C.rounding = 10 if sr else 0
+        self.Aop = self.A.T if op[0] == "t" else self.A
+        self.Bop = self.B.T if op[1] == "t" else self.B
+        self.ng = ng
+        self.flops = 2.0 * m * n * k * max(batch, 1)
+        es = np.dtype(dtype).itemsize
+        self.bytes = es * (m * k + k * n + m * n) * max(batch, 1)
+
+    def name(self):
+        return "%s%s %s m,n,k=%d,%d,%d%s%s" % ("batched%d " % self.batch if self.batch else "",
+                                                np.dtype(self.dtype).name, self.op, self.m, self.n, self.k,
+                                                " relu" if self.relu else "", " SR" if self.sr else "")
+
+    def run(self):
+        if self.batch:
+            self.ng.batched_dot(self.Aop, self.Bop, self.C, relu=self.relu)
+        else:
+            self.ng.dot(self.Aop, self.Bop, self.C, relu=self.relu)
+
+    def cpu(self):
+        a = self.hA.astype(np.float32)
+        b = self.hB.astype(np.float32)
+        a = np.swapaxes(a, -1, -2) if self.op[0] == "t" else a
+        b = np.swapaxes(b, -1, -2) if self.op[1] == "t" else b
+        import oracle as orc
+        if self.batch:
+            return orc.ref_batched_dot(a, b, relu=self.relu, acc_dtype=np.float32)
+        return orc.ref_dot(a, b, relu=self.relu, acc_dtype=np.float32)
+
+
+def time_gpu(ng, fn, iters=20, warmup=3):
+    """average duration in ms of fn() measured with HIP events on the launch stream"""
+    from nervanagpu_amd import _lib
+    for _ in range(warmup):
+        fn()
+    start, end = _lib.Event(), _lib.Event()
+    start.record(ng.stream)
+    for _ in range(iters):
+        fn()
+    end.record(ng.stream)
+    end.synchronize()
+    return end.time_since(start) / iters
+
+
+def build_config2(ng):
+    cases = []
+    for (M, K) in FC_SHAPES:
+        for op in ("nn", "nt", "tn"):
+            m, n, k = fc_mnk(op, M, K)
+            for relu in (False, True):
+                for sr in (False, True):
+                    cases.append(GemmCase(ng, op, m, n, k, relu, sr))
+    cases.append(GemmCase(ng, "nn", 4096, 4096, 4096))
+    cases.append(GemmCase(ng, "nn", 512, 512, 512, batch=32))
+    return cases
+
+
+def blas_threads():
+    try:
+        from threadpoolctl import threadpool_info
+        infos = [i for i in threadpool_info() if i.get("user_api") == "blas"]
+        if infos:
+            return int(infos[0]["num_threads"])
+    except Exception:
+        pass
+    return int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+
+
+def cpu_baseline(cases):
+    """np.dot oracle on a bounded sample of the step: one pass over the three FC
+    nn shapes plus the 4096^3 case, best of 2"""
+    sample = [c for c in cases if c.op == "nn" and not c.relu and not c.sr and not c.batch]
+    flops = sum(c.flops for c in sample)
+    best = None
+    for _ in range(2):
+        t0 = time.perf_counter()
+        for c in sample:
+            c.cpu()
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    return {"value": flops / best / 1e12, "unit": "TFLOP/s", "cores": blas_threads(), "kind": "port",
+            "sample": "np.dot (fp32 BLAS) over %s + 4096^3, one pass, best of 2; %.2f s"
+                      % (", ".join("(%d,%d)x128" % s for s in FC_SHAPES), best),
+            "host_cpus": len(os.sched_getaffinity(0))}
+
+
+# ---------------------------------------------------------------------------
+# --all: every configured case with its own roofline
+# ---------------------------------------------------------------------------
+
+ALEXNET = [(3, 224, 224, 64, 11, 11, 4, 2), (64, 27, 27, 192, 5, 5, 1, 2), (192, 13, 13, 384, 3, 3, 1, 1),
+           (384, 13, 13, 256, 3, 3, 1, 1), (256, 13, 13, 256, 3, 3, 1, 1)]
+VGG = [(3, 224, 64), (64, 224, 64), (64, 112, 128), (128, 112, 128), (128, 56, 256), (256, 56, 256),
+       (256, 28, 512), (512, 28, 512), (512, 14, 512)]
+
+
+def row(name, ms, flops=None, nbytes=None, peak_tflops=PEAK_FP16_TFLOPS):
+    r = {"case": name, "ms": ms}
+    if flops:
+        tf = flops / ms / 1e9
+        r["tflops"] = tf
+        r["pct_mfma_peak"] = 100.0 * tf / peak_tflops
+        if nbytes:
+            ceiling = min(peak_tflops, flops / nbytes * PEAK_HBM_GBS / 1e3)
+            r["pct_of_min_roof"] = 100.0 * tf / ceiling
+    if nbytes:
+        r["gbs"] = nbytes / ms / 1e6
+        if not flops:
+            r["pct_hbm_peak"] = 100.0 * r["gbs"] / PEAK_HBM_GBS
+    return r
+
+
+def conv_rows(ng, tag, N, layers, rows, iters):
+    rng = np.random.default_rng(2)
+    for cfg in layers:
+        if tag == "conv3d":
+            C, D, H, W, K, T, R, S = cfg
+            layer = ng.conv_layer(np.float16, N, C, K, D, H, W, T, R, S)
+        elif len(cfg) == 8:
+            C, H, W, K, R, S, strd, pad = cfg
+            layer = ng.conv_layer(np.float16, N, C, K, 1, H, W, 1, R, S, 0, pad, pad, 1, strd, strd)
+        else:
+            C, HW, K = cfg
+            layer = ng.conv_layer(np.float16, N, C, K, 1, HW, HW, 1, 3, 3, 0, 1, 1, 1, 1, 1)
+        I = ng.empty(layer.dimI)
+        F = ng.empty(layer.dimF)
+        E = ng.empty(layer.dimO)
+        O = ng.empty(layer.dimO)
+        B = ng.empty(layer.dimI)
+        U = ng.empty(layer.dimF, dtype=np.float32)
+        I[:] = ng.rand()
+        E[:] = ng.rand() - 0.5
+        F[:] = (ng.rand() - 0.5) * 0.05
+        sI, sF, sO = layer.sizeI * 2, layer.sizeF * 2, layer.sizeO * 2
+        nm = "%s C%d K%d %s %s" % (tag, layer.C, layer.K, layer.DHW, layer.TRS)
+        ms = time_gpu(ng, lambda: ng.fprop_conv(layer, I, F, O, relu=True), iters)
+        rows.append(row(nm + " fprop", ms, layer.flops, sI + sF + sO))
+        if tag != "conv3d":
+            ms = time_gpu(ng, lambda: ng.bprop_conv(layer, F, E, B), iters)
+            rows.append(row(nm + " bprop", ms, layer.flops, sI + sF + sO))
+            ms = time_gpu(ng, lambda: ng.update_conv(layer, I, E, U), iters)
+            rows.append(row(nm + " update", ms, layer.flops, sI + sO + layer.sizeF * 4))
+        del I, F, E, O, B, U
+
+
+def pool_rows(ng, tag, N, C, HW, win, strd, op, rows, iters):
+    layer = ng.pool_layer(np.float16, op, N, C, 1, HW, HW, 1, 1, win, win, 0, 0, 0, 0, 1, 1, strd, strd)
+    I = ng.empty(layer.dimI)
+    E = ng.empty(layer.dimO)
+    O = ng.empty(layer.dimO)
+    B = ng.empty(layer.dimI)
+    I[:] = ng.rand()
+    E[:] = ng.rand()
+    sI, sO = layer.sizeI * 2, layer.sizeO * 2
+    nm = "%s %s %dx%d/%d C%d %dx%d N%d" % (tag, op, win, win, strd, C, HW, HW, N)
+    ms = time_gpu(ng, lambda: ng.fprop_pool(layer, I, O), iters)
+    rows.append(row(nm + " fprop", ms, None, sI + sO))
+    ms = time_gpu(ng, lambda: ng.bprop_pool(layer, I, E, B), iters)
+    rows.append(row(nm + " bprop", ms, None, (2 * sI + sO) if op == "max" else (sI + sO)))
+
+
+def all_cases(ng, cases, iters=10):
+    from nervanagpu_amd import NervanaGPU
+    rows = []
+    # config 1
+    for op in ("nn", "tn"):
+        c = GemmCase(ng, op, 1024, 1024, 1024, dtype=np.float32, seed=0)
+        rows.append(row("cfg1 " + c.name(), time_gpu(ng, c.run, iters), c.flops, c.bytes, PEAK_FP32_TFLOPS))
+    # config 2
+    for c in cases:
+        if c.relu or c.sr:
+            continue
+        rows.append(row("cfg2 " + c.name(), time_gpu(ng, c.run, iters), c.flops, c.bytes))
+    for c in cases:
+        if c.sr and c.relu and c.op == "nn":
+            rows.append(row("cfg2 " + c.name(), time_gpu(ng, c.run, iters), c.flops, c.bytes))
+    conv_rows(ng, "cfg3 alexnet", 128, ALEXNET, rows, iters)
+    conv_rows(ng, "cfg4 vgg", 64, VGG, rows, iters)
+    for (C, HW) in ((64, 224), (128, 112), (256, 56), (512, 28), (512, 14)):
+        pool_rows(ng, "cfg4", 64, C, HW, 2, 2, "max", rows, iters)
+    # config 5
+    ngs = NervanaGPU(stochastic_round=True, seed=4)
+    A = ngs.empty((4096, 8192))
+    A[:] = ngs.rand()
+
+    def bn():
+        A[:] = (A - ngs.mean(A, axis=1)) / ngs.sqrt(ngs.var(A, axis=1) + 1e-3)
+    rows.append(row("cfg5 batchnorm (4096,8192) fp16 SR", time_gpu(ngs, bn, iters), None, 2 * A.nbytes))
+    Bt = ngs.empty((4096, 8192))
+    rows.append(row("cfg5 elementwise a*b+c (4096,8192) fp16",
+                    time_gpu(ngs, lambda: Bt._assign(A * A + A), iters), None, 2 * A.nbytes))
+    for op in ("max", "avg"):
+        pool_rows(ng, "cfg5", 128, 256, 56, 3, 2, op, rows, iters)
+    conv_rows(ng, "conv3d", 32, [(64, 16, 28, 28, 128, 3, 3, 3)], rows, iters)
+    return rows
+
+
+def format_rows(rows):
+    lines = ["| case | GPU ms | TFLOP/s | % MFMA peak | % of min(MFMA, AI*BW) | GB/s | % HBM peak |",
+             "|---|---|---|---|---|---|---|"]
+    for r in rows:
+        lines.append("| %s | %.4f | %s | %s | %s | %s | %s |" % (
+            r["case"], r["ms"],
+            "%.1f" % r["tflops"] if "tflops" in r else "",
+            "%.1f" % r["pct_mfma_peak"] if "pct_mfma_peak" in r else "",
+            "%.1f" % r["pct_of_min_roof"] if "pct_of_min_roof" in r else "",
+            "%.0f" % r["gbs"] if "gbs" in r else "",
+            "%.1f" % r["pct_hbm_peak"] if "pct_hbm_peak" in r else ""))
+    return "\n".join(lines)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--all", action="store_true", help="also time every configured case")
+    ap.add_argument("--out", default=None, help="file for the --all table")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (got --gpus %d); "
+                 "the data-parallel path has no collective step on one device" % args.gpus)
+
+    from nervanagpu_amd import NervanaGPU, _lib
+    ng = NervanaGPU(stochastic_round=False, bench=False, seed=1)
+    cases = build_config2(ng)
+    step_flops = sum(c.flops for c in cases)
+
+    def step():
+        for c in cases:
+            c.run()
+
+    for _ in range(args.warmup):
+        step()
+    _lib.stream_sync(ng.stream)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    _lib.stream_sync(ng.stream)
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    dominant = [c for c in cases if c.m == c.n == c.k == 4096][0]
+    dom_ms = time_gpu(ng, dominant.run, iters=max(args.steps, 20), warmup=3)
+    achieved = dominant.flops / dom_ms / 1e9
+    roofline = {"bound": "mfma", "kernel": "mfma_gemm_kernel<fp16,256x256x32,nn> (4096^3)",
+                "achieved": achieved, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                "frac": achieved / PEAK_FP16_TFLOPS, "traffic": None,
+                "launch_ms": dom_ms, "flops_per_launch": dominant.flops}
+
+    result = {
+        "metric": "fp16 GEMM/conv TFLOP/s + % MFMA peak; pool/elementwise GB/s on 1 MI355X",
+        "value": step_flops / (ms_per_step * 1e-3) / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "config 2: fp16 FC GEMM sweep N=128 (3 shapes x nn/nt/tn x relu x RN/SR) "
+                               "+ 4096^3 nn + batched 32x512^3; %d GEMM launches per step" % len(cases),
+                   "flops_per_step": step_flops},
+        "roofline": roofline,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(cases)
+
+    if args.all:
+        rows = all_cases(ng, cases)
+        table = format_rows(rows)
+        if args.out:
+            with open(args.out, "w") as f:
+                f.write(table + "\n")
+        else:
+            sys.stderr.write(table + "\n")
+        result["cases"] = rows
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
