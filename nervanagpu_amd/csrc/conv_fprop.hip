@@ -1,0 +1,70 @@
+// Convolution forward: O = round(relu?(alpha * conv(I, F))).  Replaces
+// {h,s}conv_fprop_K64_N64 (nervanagpu/nervanagpu.py:642-650, 671-734).
+#include "conv_plan.h"
+
+namespace ng {
+
+template <typename T, typename TIN, bool BLOCKED, int BM, int BN, int BK, int WM, int WN>
+static int fprop_tile(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags,
+                      hipStream_t stream)
+{
+    const ng_conv_params& p = pl.p;
+    const int ncols = p.M * p.P * p.Q * p.N;
+    const int DHWN = p.D * p.H * p.W * p.N;
+    ScaleStoreEpilogue<T> epi{(T*)O, 0, ncols, p.K, ncols, alpha, 0.0f,
+                              (flags & NG_FLAG_RELU) ? 1u : 0u, 0u, 0u, 0u, 1u};
+    PixelLattice lat{p.N, ncols, p.Q, p.P * p.Q};
+    if (BLOCKED) {
+        const int nblk = p.C / BK;
+        FilterBlockLoader<T, BK> al{(const T*)F, p.K, pl.RST * p.K, FastDiv::make((unsigned)nblk), nblk};
+        GatherColsLoader<T, TIN, true, BK> bl{(const TIN*)I, pl.d_fprop_taps, pl.CRST, lat,
+                                              p.str_d, p.str_h, p.str_w, p.D, p.H, p.W,
+                                              DHWN, FastDiv::make((unsigned)nblk), nblk};
+        return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, epi, p.K, ncols, pl.RST * nblk, 1, stream, "conv fprop");
+    } else {
+        DenseLoader<T, MC, true> al{(const T*)F, 0, p.K, p.K, pl.CRST};
+        GatherColsLoader<T, TIN, false, BK> bl{(const TIN*)I, pl.d_fprop_flat, pl.CRST, lat,
+                                               p.str_d, p.str_h, p.str_w, p.D, p.H, p.W,
+                                               0, FastDiv{0, 0}, 1};
+        return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, epi, p.K, ncols, cdiv(pl.CRST, BK), 1, stream, "conv fprop");
+    }
+}
+
+template <typename TIN, bool BLOCKED>
+static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags, hipStream_t st)
+{
+    static const int tiles[3] = {256, 128, 64};
+    switch (pick_row_tile(pl.p.K, tiles, 3)) {
+    case 256: return fprop_tile<_Float16, TIN, BLOCKED, 256, 256, 64, 2, 4>(pl, I, F, O, alpha, flags, st);
+    case 128: return fprop_tile<_Float16, TIN, BLOCKED, 128, 256, 64, 1, 4>(pl, I, F, O, alpha, flags, st);
+    default:  return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 64, 1, 4>(pl, I, F, O, alpha, flags, st);
+    }
+}
+
+}  // namespace ng
+
+using namespace ng;
+
+extern "C" int ng_conv_fprop(const void* plan, int in_dtype, const void* I, const void* F, void* O,
+                             float alpha, unsigned flags, void* /*workspace*/, size_t /*workspace_bytes*/,
+                             void* stream)
+{
+    const ConvPlan* pl = (const ConvPlan*)plan;
+    if (!pl) return fail(-48, "conv: null plan");
+    int rc;
+    if ((rc = check_ptr16(I, "I")) || (rc = check_ptr16(F, "F")) || (rc = check_ptr16(O, "O"))) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const bool blocked = pl->p.C % pl->bk == 0;
+    if (pl->dtype == NG_F16) {
+        if (in_dtype == NG_F16)
+            return blocked ? fprop_h<_Float16, true>(*pl, I, F, O, alpha, flags, st)
+                           : fprop_h<_Float16, false>(*pl, I, F, O, alpha, flags, st);
+        // byte inputs: first layers, few channels
+        if (in_dtype == NG_U8) return fprop_h<u8_t, false>(*pl, I, F, O, alpha, flags, st);
+        if (in_dtype == NG_I8) return fprop_h<s8_t, false>(*pl, I, F, O, alpha, flags, st);
+    } else if (in_dtype == NG_F32) {
+        return blocked ? fprop_tile<float, float, true, 128, 128, 16, 2, 2>(*pl, I, F, O, alpha, flags, st)
+                       : fprop_tile<float, float, false, 128, 128, 16, 2, 2>(*pl, I, F, O, alpha, flags, st);
+    }
+    return fail(-49, "conv fprop: unsupported input dtype %d for filter dtype %d", in_dtype, pl->dtype);
+}

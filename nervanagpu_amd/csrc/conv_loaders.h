@@ -1,14 +1,22 @@
 // Operand loaders and epilogues that turn the MFMA contraction core into the
 // three convolution operations on CHWN tensors (N innermost):
 //
-//   fprop   O[k, pix, n]  = sum_j  F[j, k]       * I[gather(j, pix), n]   j = (c,t,r,s)
+//   fprop   O[k, pix, n]  = sum_j  F[j, k]       * I[gather(j, pix), n]   j = (tap, c)
 //   bprop   gI[c, pix, n] = sum_j  Fs[j, c]      * E[gather(j, pix), n]   j = (tap, k)
 //   update  gF[j, k]      = sum_(pix,n) I[gather(j, pix), n] * E[k, pix, n]
 //
 // In all three the row of the activation tensor selected by (j, pix) is one
 // contiguous run of N elements, so a 16-byte chunk never straddles a pixel
-// (N is a multiple of 8) and gathers stay fully vectorised.  Which rows exist
-// is described by a small device table with one entry per contraction row j.
+// (N is a multiple of 8) and gathers stay fully vectorised.  Taps that fall
+// outside the image read as zero through the out-of-range offset of the raw
+// buffer load, so the loaders are branch free.
+//
+// "Blocked" loaders order the contraction tap-major with a whole block of BK
+// channels (fprop: input channels, bprop: output channels) per tile: the tap,
+// and with it the validity of a pixel, is uniform for a tile and the BK rows
+// differ by a constant stride.  "Flat" loaders take any row order from a table
+// with one entry per contraction row (used when the channel count is not a
+// multiple of BK, e.g. the C=3 first layers).
 //
 // Semantics follow the reference's numpy statement of the operation
 // (benchmarks/conv_test.py:99-167) and the index formulas of
@@ -19,45 +27,70 @@
 
 namespace ng {
 
-// one contraction row: element offset of the tap relative to the pixel origin,
-// and the tap's coordinate deltas for the bounds test
+// a tap (or, in flat tables, one contraction row): element offset relative to
+// the pixel origin and the coordinate deltas for the bounds test
 struct TapEntry { int off, dz, dy, dx; };
 
 typedef unsigned char u8_t;
 typedef signed char   s8_t;
 
-// 16-byte chunk of compute type T from a run of storage type TIN
+// n / d for 0 <= n < 2^31 as a multiply and a shift.  With s = ceil(log2 d),
+// mul = floor(2^(31+s) / d) + 1 fits 32 bits and the quotient is exact because
+// the rounding excess n * (mul*d - 2^(31+s)) stays below 2^(31+s).
+struct FastDiv {
+    unsigned mul, shift;
+    __host__ __device__ __forceinline__ unsigned div(unsigned n) const
+    {
+        return (unsigned)(((unsigned long long)n * mul) >> shift);
+    }
+    static FastDiv make(unsigned d)
+    {
+        unsigned s = 0;
+        while ((1ull << s) < d) s++;
+        FastDiv f;
+        f.mul = (unsigned)((1ull << (31 + s)) / d + 1);
+        f.shift = 31 + s;
+        return f;
+    }
+};
+
+// 16-byte chunk of compute type T from storage type TIN via a raw buffer load
 template <typename T, typename TIN> struct ChunkFetch;
 
 template <typename T> struct ChunkFetch<T, T> {
-    static __device__ __forceinline__ uint4_t get(const T* p) { return *reinterpret_cast<const uint4_t*>(p); }
+    static constexpr int ES = (int)sizeof(T);
+    static __device__ __forceinline__ uint4_t get(BufferRsrc r, unsigned byte_off) { return buffer_load_chunk(r, byte_off); }
 };
 
 // bytes -> fp16, exact for every 8-bit value (I2F on load in the reference,
 // kernels/sass/hconv_updat_C64_K64.sass:324-345)
 template <> struct ChunkFetch<_Float16, u8_t> {
-    static __device__ __forceinline__ uint4_t get(const u8_t* p)
+    static constexpr int ES = 1;
+    static __device__ __forceinline__ uint4_t get(BufferRsrc r, unsigned byte_off)
     {
-        const uint2 raw = *reinterpret_cast<const uint2*>(p);
+        typedef unsigned uint2_t __attribute__((ext_vector_type(2)));
+        const uint2_t raw = __builtin_amdgcn_raw_buffer_load_b64(r, (int)byte_off, 0, 0);
         _Float16 h[8];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            h[e]     = (_Float16)(float)((raw.x >> (8 * e)) & 0xFFu);
-            h[e + 4] = (_Float16)(float)((raw.y >> (8 * e)) & 0xFFu);
+            h[e]     = (_Float16)(float)((raw[0] >> (8 * e)) & 0xFFu);
+            h[e + 4] = (_Float16)(float)((raw[1] >> (8 * e)) & 0xFFu);
         }
         return *reinterpret_cast<const uint4_t*>(h);
     }
 };
 
 template <> struct ChunkFetch<_Float16, s8_t> {
-    static __device__ __forceinline__ uint4_t get(const s8_t* p)
+    static constexpr int ES = 1;
+    static __device__ __forceinline__ uint4_t get(BufferRsrc r, unsigned byte_off)
     {
-        const uint2 raw = *reinterpret_cast<const uint2*>(p);
+        typedef unsigned uint2_t __attribute__((ext_vector_type(2)));
+        const uint2_t raw = __builtin_amdgcn_raw_buffer_load_b64(r, (int)byte_off, 0, 0);
         _Float16 h[8];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            h[e]     = (_Float16)(float)(int)(signed char)((raw.x >> (8 * e)) & 0xFFu);
-            h[e + 4] = (_Float16)(float)(int)(signed char)((raw.y >> (8 * e)) & 0xFFu);
+            h[e]     = (_Float16)(float)(int)(signed char)((raw[0] >> (8 * e)) & 0xFFu);
+            h[e + 4] = (_Float16)(float)(int)(signed char)((raw[1] >> (8 * e)) & 0xFFu);
         }
         return *reinterpret_cast<const uint4_t*>(h);
     }
@@ -71,80 +104,176 @@ struct PixelLattice {
     int nx, nxy;    // nx, nx*ny
 };
 
+#define NG_FAR (-0x40000000)
+
 // B operand of fprop / bprop (row-contiguous tile: lines are contraction rows,
-// columns are (pixel, n)).  Gathered coordinate of tap j at lattice point
-// (iz,iy,ix) is (iz*gs_d + dz_j, iy*gs_h + dy_j, ix*gs_w + dx_j) inside a
-// (lim_d, lim_h, lim_w) volume; taps outside contribute zero.
-template <typename T, typename TIN>
+// columns are (pixel, n)).  Gathered coordinate of a tap at lattice point
+// (iz,iy,ix) is (iz*gs_d + dz, iy*gs_h + dy, ix*gs_w + dx) inside a
+// (lim_d, lim_h, lim_w) volume.
+template <typename T, typename TIN, bool BLOCKED, int BK>
 struct GatherColsLoader {
     const TIN*      X;
-    const TapEntry* tab;
+    const TapEntry* tab;        // BLOCKED: one entry per tap; flat: one per contraction row
     int             J;          // contraction rows
     PixelLattice    lat;
     int             gs_d, gs_h, gs_w;
     int             lim_d, lim_h, lim_w;
+    int             row_stride; // BLOCKED: elements between consecutive rows of a block
+    FastDiv         blk_div;    // BLOCKED: tile index -> tap (blocks per tap = nblk)
+    int             nblk;
 
-    struct Ctx { int base, z0, y0, x0; };
+    struct Ctx { int base, z0, y0, x0, kr; };
+    struct Tile { BufferRsrc rsrc; int toff, dz, dy, dx, k0; };
 
-    __device__ __forceinline__ Ctx prepare(int col) const
+    __device__ __forceinline__ Ctx prepare(int col, int kr) const
     {
         Ctx c;
-        if (col >= lat.ncols) { c.base = 0; c.z0 = c.y0 = c.x0 = -0x40000000; return c; }
+        c.kr = kr;
+        if (col >= lat.ncols) { c.base = 0; c.z0 = c.y0 = c.x0 = NG_FAR; return c; }
         const int pix = col / lat.N, nn = col - pix * lat.N;
         const int iz = pix / lat.nxy, rem = pix - iz * lat.nxy;
         const int iy = rem / lat.nx, ix = rem - iy * lat.nx;
         c.z0 = iz * gs_d; c.y0 = iy * gs_h; c.x0 = ix * gs_w;
         c.base = ((c.z0 * lim_h + c.y0) * lim_w + c.x0) * lat.N + nn;
+        if (BLOCKED) c.base += kr * row_stride;
         return c;
     }
 
-    __device__ __forceinline__ uint4_t load(const Ctx& c, int k, int /*zb*/) const
+    __device__ __forceinline__ Tile tile(int kt, int k0, int /*zb*/) const
     {
-        uint4_t out = {0u, 0u, 0u, 0u};
-        if (k < J) {
-            const TapEntry e = tab[k];
-            if ((unsigned)(c.z0 + e.dz) < (unsigned)lim_d && (unsigned)(c.y0 + e.dy) < (unsigned)lim_h &&
-                (unsigned)(c.x0 + e.dx) < (unsigned)lim_w)
-                out = ChunkFetch<T, TIN>::get(X + (c.base + e.off));
+        Tile t;
+        t.rsrc = make_rsrc(X);
+        t.k0 = k0;
+        if (BLOCKED) {
+            const int tap = (int)blk_div.div((unsigned)kt);
+            const int blk = kt - tap * nblk;
+            const TapEntry e = tab[tap];
+            t.toff = e.off + blk * BK * row_stride;
+            t.dz = e.dz; t.dy = e.dy; t.dx = e.dx;
+        } else {
+            t.toff = 0; t.dz = t.dy = t.dx = 0;
         }
-        return out;
+        return t;
+    }
+
+    __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const
+    {
+        constexpr int ES = ChunkFetch<T, TIN>::ES;
+        if (BLOCKED) {
+            const bool ok = (unsigned)(c.z0 + t.dz) < (unsigned)lim_d && (unsigned)(c.y0 + t.dy) < (unsigned)lim_h &&
+                            (unsigned)(c.x0 + t.dx) < (unsigned)lim_w;
+            return ChunkFetch<T, TIN>::get(t.rsrc, ok ? (unsigned)(c.base + t.toff) * ES : NG_OOB_OFFSET);
+        } else {
+            const int k = t.k0 + c.kr;
+            const TapEntry e = tab[min(k, J - 1)];
+            const bool ok = k < J && (unsigned)(c.z0 + e.dz) < (unsigned)lim_d &&
+                            (unsigned)(c.y0 + e.dy) < (unsigned)lim_h && (unsigned)(c.x0 + e.dx) < (unsigned)lim_w;
+            return ChunkFetch<T, TIN>::get(t.rsrc, ok ? (unsigned)(c.base + e.off) * ES : NG_OOB_OFFSET);
+        }
     }
 };
 
+// A operand of blocked fprop: filter F[c][tap][k] read as rows j = (tap, c):
+// tile (tap, block) holds channels block*BK .. +BK-1, consecutive rows are
+// RST*K elements apart.
+template <typename T, int BK>
+struct FilterBlockLoader {
+    const T* F;
+    int      K;          // row length (output feature maps)
+    int      RSTK;       // elements between consecutive channels
+    FastDiv  blk_div;
+    int      nblk;
+
+    struct Ctx { unsigned off; };
+    struct Tile { BufferRsrc rsrc; };
+
+    __device__ __forceinline__ Ctx prepare(int m, int kr) const
+    {
+        Ctx c;
+        c.off = (m < K) ? (unsigned)(kr * RSTK + m) * (unsigned)sizeof(T) : NG_OOB_OFFSET;
+        return c;
+    }
+    __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/) const
+    {
+        const int tap = (int)blk_div.div((unsigned)kt);
+        const int blk = kt - tap * nblk;
+        Tile t;
+        t.rsrc = make_rsrc(F + (long)blk * BK * RSTK + (long)tap * K);
+        return t;
+    }
+    __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const { return buffer_load_chunk(t.rsrc, c.off); }
+};
+
 // A operand of update (contraction-contiguous tile: rows are filter rows
-// j = (c,t,r,s), the contraction index is (output pixel, n)).
-template <typename T, typename TIN>
+// j = (c,t,r,s), the contraction index is (output pixel, n)).  BLOCKED: N is a
+// multiple of BK, so a tile lies inside one output pixel.
+template <typename T, typename TIN, bool BLOCKED, int BK>
 struct GatherRowsLoader {
     const TIN*      X;
-    const TapEntry* tab;
+    const TapEntry* tab;        // one entry per filter row
     int             J;          // filter rows C*T*R*S
     int             N, kdim;    // kdim = M*P*Q*N
     int             Q, PQ;
     int             str_d, str_h, str_w;
     int             D, H, W;
+    FastDiv         npt_div, pq_div, q_div;   // tiles per pixel, P*Q, Q
+    int             npt;
 
-    typedef TapEntry Ctx;
+    struct Ctx { int off, dz, dy, dx, kc; };
+    struct Tile { BufferRsrc rsrc; int pixbase, z0, y0, x0, k0; };
 
-    __device__ __forceinline__ Ctx prepare(int r) const
+    __device__ __forceinline__ Ctx prepare(int r, int kc) const
     {
-        if (r < J) return tab[r];
-        Ctx c = {0, -0x40000000, -0x40000000, -0x40000000};
+        Ctx c;
+        c.kc = kc;
+        if (r < J) {
+            const TapEntry e = tab[r];
+            c.off = e.off + (BLOCKED ? kc : 0); c.dz = e.dz; c.dy = e.dy; c.dx = e.dx;
+        } else {
+            c.off = 0; c.dz = c.dy = c.dx = NG_FAR;
+        }
         return c;
     }
 
-    __device__ __forceinline__ uint4_t load(const Ctx& c, int kk, int /*zb*/) const
+    __device__ __forceinline__ Tile tile(int kt, int k0, int /*zb*/) const
     {
-        uint4_t out = {0u, 0u, 0u, 0u};
-        if (kk < kdim) {
-            const int pix = kk / N, nn = kk - pix * N;
+        Tile t;
+        t.rsrc = make_rsrc(X);
+        t.k0 = k0;
+        if (BLOCKED) {
+            const unsigned pix = npt_div.div((unsigned)kt);
+            const int nb = kt - (int)pix * npt;
+            const unsigned m = pq_div.div(pix);
+            const unsigned rem = pix - m * PQ;
+            const unsigned p = q_div.div(rem);
+            const unsigned q = rem - p * Q;
+            t.z0 = (int)m * str_d; t.y0 = (int)p * str_h; t.x0 = (int)q * str_w;
+            t.pixbase = ((t.z0 * H + t.y0) * W + t.x0) * N + nb * BK;
+        } else {
+            t.z0 = t.y0 = t.x0 = t.pixbase = 0;
+        }
+        return t;
+    }
+
+    __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const
+    {
+        constexpr int ES = ChunkFetch<T, TIN>::ES;
+        if (BLOCKED) {
+            const bool ok = (unsigned)(t.z0 + c.dz) < (unsigned)D && (unsigned)(t.y0 + c.dy) < (unsigned)H &&
+                            (unsigned)(t.x0 + c.dx) < (unsigned)W;
+            return ChunkFetch<T, TIN>::get(t.rsrc, ok ? (unsigned)(t.pixbase + c.off) * ES : NG_OOB_OFFSET);
+        } else {
+            const int kk = t.k0 + c.kc;
+            const int kc2 = min(kk, kdim - 1);
+            const int pix = kc2 / N, nn = kc2 - pix * N;
             const int m = pix / PQ, rem = pix - m * PQ;
             const int p = rem / Q, q = rem - p * Q;
             const int z0 = m * str_d, y0 = p * str_h, x0 = q * str_w;
-            if ((unsigned)(z0 + c.dz) < (unsigned)D && (unsigned)(y0 + c.dy) < (unsigned)H &&
-                (unsigned)(x0 + c.dx) < (unsigned)W)
-                out = ChunkFetch<T, TIN>::get(X + (((z0 * H + y0) * W + x0) * N + nn + c.off));
+            const bool ok = kk < kdim && (unsigned)(z0 + c.dz) < (unsigned)D && (unsigned)(y0 + c.dy) < (unsigned)H &&
+                            (unsigned)(x0 + c.dx) < (unsigned)W;
+            return ChunkFetch<T, TIN>::get(
+                t.rsrc, ok ? (unsigned)(((z0 * H + y0) * W + x0) * N + nn + c.off) * ES : NG_OOB_OFFSET);
         }
-        return out;
     }
 };
 

@@ -1,0 +1,84 @@
+// Host-side description of one convolution geometry, shared by the three
+// convolution translation units.
+#pragma once
+
+#include "conv_loaders.h"
+
+#include <algorithm>
+#include <vector>
+
+namespace ng {
+
+struct BpropClass {
+    int rz, ry, rx;         // residues of the input pixel coordinates
+    int nz, ny, nx;         // lattice extents of the class
+    int taps;               // filter taps that reach the class
+    int J;                  // contraction rows: taps * K
+    long flat_offset;       // first flat TapEntry (one per (tap,k)) in d_bprop_flat
+    long tap_offset;        // first per-tap TapEntry in d_bprop_taps
+    long w_row;             // first row of the class in the re-laid filter
+};
+
+struct ConvPlan {
+    ng_conv_params p;
+    int dtype;
+    int bk;                 // contraction tile depth of the kernels for this dtype
+    int CRST, RST, Cpad;
+    TapEntry* d_fprop_flat = nullptr;   // CRST entries, rows (c,t,r,s)
+    TapEntry* d_fprop_taps = nullptr;   // RST entries
+    TapEntry* d_bprop_flat = nullptr;   // K*RST entries grouped by class, rows (tap,k)
+    TapEntry* d_bprop_taps = nullptr;   // RST entries grouped by class
+    int* d_tap_dest = nullptr;          // RST ints: first re-laid filter row of each tap
+    std::vector<BpropClass> classes;
+    size_t ws_bprop = 0, ws_update = 0;
+};
+
+inline int cdiv(int a, int b) { return (a + b - 1) / b; }
+
+// how many slices to cut a contraction into so that the grid fills the chip
+inline int conv_splits(int out_tiles, int total_k_tiles, size_t slice_bytes, size_t ws_bytes)
+{
+    const int cus = device_cu_count();
+    if (out_tiles >= cus || total_k_tiles < 8) return 1;
+    int splits = cdiv(cus, out_tiles);
+    splits = std::min(splits, total_k_tiles / 4);
+    if (slice_bytes) splits = (int)std::min<size_t>((size_t)splits, ws_bytes / slice_bytes);
+    while (splits > 1 && (splits - 1) * cdiv(total_k_tiles, splits) >= total_k_tiles) splits--;
+    return std::max(splits, 1);
+}
+
+inline int check_ptr16(const void* p, const char* what)
+{
+    if (!p) return fail(-41, "conv: null %s", what);
+    if ((uintptr_t)p & 15) return fail(-42, "conv: %s must be 16-byte aligned", what);
+    return 0;
+}
+
+// row tile (output feature maps or input channels) with the least padding
+inline int pick_row_tile(int rows, const int* tiles, int n)
+{
+    int best = tiles[0], best_pad = cdiv(rows, best) * best;
+    for (int i = 1; i < n; i++) {
+        const int pad = cdiv(rows, tiles[i]) * tiles[i];
+        if (pad < best_pad) { best = tiles[i]; best_pad = pad; }
+    }
+    return best;
+}
+
+template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, class AL, class BL, class Epi>
+inline int launch_core(const AL& al, const BL& bl, const Epi& epi, int rows, int ncols, int k_tiles, int splits,
+                       hipStream_t stream, const char* what)
+{
+    CoreShape s;
+    s.m = rows; s.n = ncols;
+    s.k_tiles = k_tiles;
+    s.passes = 1; s.splits = splits;
+    s.tiles_m = cdiv(rows, BM);
+    s.tiles_n = cdiv(ncols, BN);
+    hipLaunchKernelGGL((mfma_gemm_kernel<T, BM, BN, BK, WM, WN, LA, LB, AL, BL, Epi>),
+                       dim3(s.tiles_m * s.tiles_n, splits, 1), dim3(WM * WN * 64), 0, stream, al, bl, epi, s);
+    NG_CHECK_LAUNCH(what);
+    return 0;
+}
+
+}  // namespace ng

@@ -1,0 +1,129 @@
+// Convolution plans: the per-geometry tap tables of the gather loaders
+// (counterpart of ConvLayer.__init__ precomputing its kernel arguments,
+// nervanagpu/layers.py:281-481).
+#include "conv_plan.h"
+
+using namespace ng;
+
+extern "C" {
+
+int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
+{
+    *plan_out = nullptr;
+    const ng_conv_params& p = *pp;
+    if (dtype != NG_F16 && dtype != NG_F32) return fail(-43, "conv: dtype must be fp16 or fp32");
+    if (p.N % 8 || p.K % 8) return fail(-44, "conv: N and K must be multiples of 8");
+    if (p.N <= 0 || p.C <= 0 || p.K <= 0 || p.M <= 0 || p.P <= 0 || p.Q <= 0) return fail(-45, "conv: empty geometry");
+    if (p.str_d < 1 || p.str_h < 1 || p.str_w < 1) return fail(-46, "conv: strides must be >= 1");
+    const long sizeI = (long)p.C * p.D * p.H * p.W * p.N, sizeO = (long)p.K * p.M * p.P * p.Q * p.N;
+    const long es = (long)dtype_size(dtype);
+    if (sizeI * es >= (1L << 31) || sizeO * es >= (1L << 31))
+        return fail(-47, "conv: tensors of 2 GiB or more are not supported");
+
+    ConvPlan* pl = new ConvPlan();
+    pl->p = p;
+    pl->dtype = dtype;
+    pl->bk = (dtype == NG_F16) ? 64 : 16;
+    pl->RST = p.T * p.R * p.S;
+    pl->CRST = p.C * pl->RST;
+    pl->Cpad = cdiv(p.C, 8) * 8;
+    const int HW = p.H * p.W, DHW = p.D * HW;
+
+    // forward taps
+    std::vector<TapEntry> ftaps((size_t)pl->RST), fflat((size_t)pl->CRST);
+    for (int t = 0; t < p.T; t++)
+        for (int r = 0; r < p.R; r++)
+            for (int s = 0; s < p.S; s++) {
+                const int dz = t - p.pad_d, dy = r - p.pad_h, dx = s - p.pad_w;
+                const int trs = (t * p.R + r) * p.S + s;
+                ftaps[(size_t)trs] = TapEntry{(int)(((long)dz * HW + dy * p.W + dx) * p.N), dz, dy, dx};
+                for (int c = 0; c < p.C; c++)
+                    fflat[(size_t)c * pl->RST + trs] =
+                        TapEntry{(int)(((long)c * DHW + (long)dz * HW + dy * p.W + dx) * p.N), dz, dy, dx};
+            }
+
+    // data-gradient classes: input pixel (z,y,x) with z % str_d == rz ... receives
+    // tap t iff (rz + pad_d - t) % str_d == 0, from output m = iz + (rz + pad_d - t)/str_d
+    std::vector<TapEntry> bflat, btaps;
+    std::vector<int> tap_dest((size_t)pl->RST, 0);
+    const int PQ = p.P * p.Q;
+    long w_row = 0;
+    for (int rz = 0; rz < p.str_d; rz++)
+        for (int ry = 0; ry < p.str_h; ry++)
+            for (int rx = 0; rx < p.str_w; rx++) {
+                BpropClass c;
+                c.rz = rz; c.ry = ry; c.rx = rx;
+                c.nz = (p.D > rz) ? (p.D - rz + p.str_d - 1) / p.str_d : 0;
+                c.ny = (p.H > ry) ? (p.H - ry + p.str_h - 1) / p.str_h : 0;
+                c.nx = (p.W > rx) ? (p.W - rx + p.str_w - 1) / p.str_w : 0;
+                c.flat_offset = (long)bflat.size();
+                c.tap_offset = (long)btaps.size();
+                c.w_row = w_row;
+                int taps = 0;
+                for (int t = 0; t < p.T; t++) {
+                    if ((rz + p.pad_d - t) % p.str_d) continue;
+                    for (int r = 0; r < p.R; r++) {
+                        if ((ry + p.pad_h - r) % p.str_h) continue;
+                        for (int s = 0; s < p.S; s++) {
+                            if ((rx + p.pad_w - s) % p.str_w) continue;
+                            const int dz = (rz + p.pad_d - t) / p.str_d, dy = (ry + p.pad_h - r) / p.str_h,
+                                      dx = (rx + p.pad_w - s) / p.str_w;
+                            tap_dest[(size_t)(t * p.R + r) * p.S + s] = (int)(w_row + (long)taps * p.K);
+                            btaps.push_back(TapEntry{(int)(((long)dz * PQ + dy * p.Q + dx) * p.N), dz, dy, dx});
+                            for (int k = 0; k < p.K; k++)
+                                bflat.push_back(TapEntry{(int)(((long)k * p.M * PQ + (long)dz * PQ + dy * p.Q + dx) * p.N),
+                                                         dz, dy, dx});
+                            taps++;
+                        }
+                    }
+                }
+                c.taps = taps;
+                c.J = taps * p.K;
+                w_row += c.J;
+                pl->classes.push_back(c);
+            }
+
+    auto upload = [&](const void* src, size_t bytes, void** dst) -> int {
+        if (bytes == 0) { *dst = nullptr; return 0; }
+        NG_HIP(hipMalloc(dst, bytes));
+        NG_HIP(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
+        return 0;
+    };
+    int rc = upload(fflat.data(), fflat.size() * sizeof(TapEntry), (void**)&pl->d_fprop_flat);
+    if (!rc) rc = upload(ftaps.data(), ftaps.size() * sizeof(TapEntry), (void**)&pl->d_fprop_taps);
+    if (!rc) rc = upload(bflat.data(), bflat.size() * sizeof(TapEntry), (void**)&pl->d_bprop_flat);
+    if (!rc) rc = upload(btaps.data(), btaps.size() * sizeof(TapEntry), (void**)&pl->d_bprop_taps);
+    if (!rc) rc = upload(tap_dest.data(), tap_dest.size() * sizeof(int), (void**)&pl->d_tap_dest);
+    if (rc) { ng_conv_plan_destroy(pl); return rc; }
+
+    pl->ws_bprop = align_up((size_t)pl->RST * p.K * pl->Cpad * dtype_size(dtype), 256);
+    {
+        const int kt = cdiv(p.M * p.P * p.Q * p.N, pl->bk);
+        const int tiles = cdiv(pl->CRST, 128) * cdiv(p.K, 128);
+        const int splits = conv_splits(tiles, kt, 0, 0);
+        pl->ws_update = splits > 1 ? align_up((size_t)splits * pl->CRST * p.K * sizeof(float), 256) : 0;
+    }
+    *plan_out = pl;
+    return 0;
+}
+
+int ng_conv_plan_destroy(void* plan)
+{
+    ConvPlan* pl = (ConvPlan*)plan;
+    if (!pl) return 0;
+    if (pl->d_fprop_flat) (void)hipFree(pl->d_fprop_flat);
+    if (pl->d_fprop_taps) (void)hipFree(pl->d_fprop_taps);
+    if (pl->d_bprop_flat) (void)hipFree(pl->d_bprop_flat);
+    if (pl->d_bprop_taps) (void)hipFree(pl->d_bprop_taps);
+    if (pl->d_tap_dest) (void)hipFree(pl->d_tap_dest);
+    delete pl;
+    return 0;
+}
+
+size_t ng_conv_plan_workspace_bytes(const void* plan)
+{
+    const ConvPlan* pl = (const ConvPlan*)plan;
+    return pl ? std::max(pl->ws_bprop, pl->ws_update) : 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,76 @@
+// Convolution weight gradient: gradF = round(alpha * sum_{pixels,n} I x E).
+// Replaces {h,s}conv_updat_C128_{K64,K128}, the zero fill and the fp32 convert
+// launch (nervanagpu/nervanagpu.py:661-669, 695-724).  fp32 partial sums over
+// slices of the (pixel, n) range are added in a fixed order instead of with
+// fp32 atomics, so the result does not depend on execution order.
+#include "conv_plan.h"
+
+namespace ng {
+
+template <typename T, typename TIN, typename TOUT, bool BLOCKED, int BM, int BN, int BK, int WM, int WN>
+static int launch_update(const ConvPlan& pl, const void* I, const void* E, void* gradF, float alpha,
+                         void* ws, size_t ws_bytes, hipStream_t stream)
+{
+    const ng_conv_params& p = pl.p;
+    const int kdim = p.M * p.P * p.Q * p.N;
+    const int rows = pl.CRST, cols = p.K;
+    const int k_tiles = cdiv(kdim, BK);
+    const int tiles = cdiv(rows, BM) * cdiv(cols, BN);
+    const size_t slice = (size_t)rows * cols * sizeof(float);
+    const int splits = ws ? conv_splits(tiles, k_tiles, slice, ws_bytes) : 1;
+    const int npt = BLOCKED ? p.N / BK : 1;
+
+    GatherRowsLoader<T, TIN, BLOCKED, BK> al{(const TIN*)I, pl.d_fprop_flat, pl.CRST, p.N, kdim, p.Q, p.P * p.Q,
+                                             p.str_d, p.str_h, p.str_w, p.D, p.H, p.W,
+                                             FastDiv::make((unsigned)npt), FastDiv::make((unsigned)(p.P * p.Q)),
+                                             FastDiv::make((unsigned)p.Q), npt};
+    DenseLoader<T, KC, true> bl{(const T*)E, 0, kdim, p.K, kdim};
+    ScaleStoreEpilogue<TOUT> epi{(TOUT*)gradF, 0, p.K, rows, cols, alpha, 0.0f, 0u, 0u, 0u, 0u,
+                                 (((uintptr_t)gradF & 15) == 0) ? 1u : 0u};
+    if (splits == 1)
+        return launch_core<T, BM, BN, BK, WM, WN, KC, KC>(al, bl, epi, rows, cols, k_tiles, 1, stream, "conv update");
+    PartialEpilogue pe{(float*)ws, rows, cols, 1, 1u};
+    int rc = launch_core<T, BM, BN, BK, WM, WN, KC, KC>(al, bl, pe, rows, cols, k_tiles, splits, stream, "conv update");
+    if (rc) return rc;
+    const long total = (long)rows * cols;
+    const int blocks = (int)std::min<long>((total + 255) / 256, 8192);
+    hipLaunchKernelGGL((splitk_reduce_kernel<TOUT, ScaleStoreEpilogue<TOUT>>), dim3(blocks), dim3(256), 0,
+                       stream, (const float*)ws, splits, 1, rows, cols, epi);
+    NG_CHECK_LAUNCH("conv update reduce");
+    return 0;
+}
+
+template <typename TIN, typename TOUT>
+static int update_h(const ConvPlan& pl, const void* I, const void* E, void* gradF, float alpha,
+                    void* ws, size_t ws_bytes, hipStream_t st)
+{
+    if (pl.p.N % 64 == 0)
+        return launch_update<_Float16, TIN, TOUT, true, 128, 128, 64, 2, 2>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
+    return launch_update<_Float16, TIN, TOUT, false, 128, 128, 64, 2, 2>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
+}
+
+}  // namespace ng
+
+using namespace ng;
+
+extern "C" int ng_conv_update(const void* plan, int in_dtype, int out_dtype, const void* I, const void* E,
+                              void* gradF, float alpha, void* workspace, size_t workspace_bytes, void* stream)
+{
+    const ConvPlan* pl = (const ConvPlan*)plan;
+    if (!pl) return fail(-48, "conv: null plan");
+    int rc;
+    if ((rc = check_ptr16(I, "I")) || (rc = check_ptr16(E, "E")) || (rc = check_ptr16(gradF, "grad_F"))) return rc;
+    if (workspace && ((uintptr_t)workspace & 15)) return fail(-42, "conv: workspace must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    if (pl->dtype == NG_F16) {
+        if (in_dtype == NG_F16 && out_dtype == NG_F32) return update_h<_Float16, float>(*pl, I, E, gradF, alpha, workspace, workspace_bytes, st);
+        if (in_dtype == NG_F16 && out_dtype == NG_F16) return update_h<_Float16, _Float16>(*pl, I, E, gradF, alpha, workspace, workspace_bytes, st);
+        if (in_dtype == NG_U8 && out_dtype == NG_F32)  return update_h<u8_t, float>(*pl, I, E, gradF, alpha, workspace, workspace_bytes, st);
+        if (in_dtype == NG_U8 && out_dtype == NG_F16)  return update_h<u8_t, _Float16>(*pl, I, E, gradF, alpha, workspace, workspace_bytes, st);
+    } else if (in_dtype == NG_F32 && out_dtype == NG_F32) {
+        if (pl->p.N % 16 == 0)
+            return launch_update<float, float, float, true, 128, 128, 16, 2, 2>(*pl, I, E, gradF, alpha, workspace, workspace_bytes, st);
+        return launch_update<float, float, float, false, 128, 128, 16, 2, 2>(*pl, I, E, gradF, alpha, workspace, workspace_bytes, st);
+    }
+    return fail(-50, "conv update: unsupported dtype combination (in %d, out %d, filter %d)", in_dtype, out_dtype, pl->dtype);
+}

@@ -92,11 +92,14 @@ template <typename T>
 static bool operands_vectorizable(const GemmArgs& g)
 {
     constexpr int EPC = Elem<T>::EPC;
-    auto ok = [&](const void* p, int ld, long ldz, int contiguous_extent) {
-        return ((uintptr_t)p & 15) == 0 && ld % EPC == 0 && ldz % EPC == 0 && contiguous_extent % EPC == 0;
+    // 16-byte chunks must be aligned and whole, and one matrix must fit the
+    // 2 GiB window of a buffer descriptor
+    auto ok = [&](const void* p, int ld, long ldz, int contiguous_extent, int other_extent) {
+        return ((uintptr_t)p & 15) == 0 && ld % EPC == 0 && ldz % EPC == 0 && contiguous_extent % EPC == 0 &&
+               (long)other_extent * ld * (long)sizeof(T) < (1L << 31);
     };
-    const bool a = ok(g.A, g.lda, g.ldaz, g.trans_a ? g.m : g.k);
-    const bool b = ok(g.B, g.ldb, g.ldbz, g.trans_b ? g.k : g.n);
+    const bool a = ok(g.A, g.lda, g.ldaz, g.trans_a ? g.m : g.k, g.trans_a ? g.k : g.m);
+    const bool b = ok(g.B, g.ldb, g.ldbz, g.trans_b ? g.k : g.n, g.trans_b ? g.n : g.k);
     return a && b;
 }
 
@@ -108,12 +111,9 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
     const bool vec = operands_vectorizable<_Float16>(g);
     const long big_tiles = (long)ceil_div(g.m, 256) * ceil_div(g.n, 256) * g.batch_grid;
     const bool large = g.m >= 256 && g.n >= 256 && big_tiles >= device_cu_count() / 2;
-    if (large) {
-        return vec ? launch_layout<_Float16, 256, 256, 32, 2, 2, true>(g, sr_bits)
-                   : launch_layout<_Float16, 256, 256, 32, 2, 2, false>(g, sr_bits);
-    }
-    return vec ? launch_layout<_Float16, 128, 128, 32, 2, 2, true>(g, sr_bits)
-               : launch_layout<_Float16, 128, 128, 32, 2, 2, false>(g, sr_bits);
+    if (large && vec) return launch_layout<_Float16, 256, 256, 64, 2, 4, true>(g, sr_bits);
+    return vec ? launch_layout<_Float16, 128, 128, 64, 2, 2, true>(g, sr_bits)
+               : launch_layout<_Float16, 128, 128, 64, 2, 2, false>(g, sr_bits);
 }
 
 template <>
@@ -157,7 +157,7 @@ size_t ng_gemm_workspace_bytes(int dtype, int trans_a, int trans_b, int m, int n
                                int batch_grid, int batch_loops)
 {
     (void)trans_a; (void)trans_b;
-    const int bk = (dtype == NG_F16) ? 32 : 16;
+    const int bk = (dtype == NG_F16) ? 64 : 16;
     const int bt = 128;
     const int out_tiles = ceil_div(m, bt) * ceil_div(n, bt) * batch_grid;
     const int total_k = ceil_div(k, bk) * batch_loops;

@@ -141,9 +141,38 @@ struct CoreShape {
     int tiles_m, tiles_n;
 };
 
+// Global operand chunks are fetched with raw buffer loads: an offset at or
+// beyond the 2 GiB range of the descriptor returns zeros in hardware, which is
+// how invalid rows, contraction tails and out-of-image convolution taps become
+// zero operands without a branch or a select after the load.
+typedef __amdgpu_buffer_rsrc_t BufferRsrc;
+#define NG_OOB_OFFSET 0x80000000u
+
+__device__ __forceinline__ BufferRsrc make_rsrc(const void* base)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x80000000, 0x00020000);
+}
+
+__device__ __forceinline__ uint4_t buffer_load_chunk(BufferRsrc rsrc, unsigned byte_offset)
+{
+    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)byte_offset, 0, 0);
+}
+
+// Loader protocol used by the core (all three calls are inlined):
+//   Ctx  prepare(r, kc)      once per 16-byte chunk a thread owns: r = absolute
+//                            row of the operand, kc = contraction offset of the
+//                            chunk inside a tile
+//   Tile tile(kt, k0, zb)    once per contraction tile, wavefront-uniform values
+//                            (kt = tile index inside the pass, k0 = kt*BK,
+//                            zb = batch / pass index)
+//   load(tile, ctx)          the chunk; must be branch free so that the loads of
+//                            the next tile can be scheduled between the MFMAs of
+//                            the current one
+//
 // Dense row-major operand.  KC: element (r,k) at base[r*ld + k]; MC: at base[k*ld + r].
-// VEC: the host guarantees 16-byte alignment of every chunk and that chunks do
-// not straddle the matrix edge; otherwise elements are fetched one by one.
+// VEC: the host guarantees 16-byte alignment of every chunk, that chunks do not
+// straddle the matrix edge and that the matrix spans less than 4 GiB; otherwise
+// elements are fetched one by one.
 template <typename T, int LAYOUT, bool VEC>
 struct DenseLoader {
     const T* base;
@@ -152,32 +181,48 @@ struct DenseLoader {
     int      rows;   // extent along r
     int      kdim;   // extent along k (per pass)
 
-    typedef int Ctx;   // per-chunk row context: the row index itself
-    __device__ __forceinline__ Ctx prepare(int r) const { return r; }
+    struct Ctx { unsigned off; int k; int r; };
+    struct Tile { BufferRsrc rsrc; const T* p; int krem; };
 
-    __device__ __forceinline__ uint4_t load(const Ctx& r, int k, int zb) const
+    __device__ __forceinline__ Ctx prepare(int r, int kc) const
+    {
+        Ctx c;
+        c.k = kc;
+        c.r = r;
+        const unsigned e = (LAYOUT == KC) ? (unsigned)r * (unsigned)ld + (unsigned)kc
+                                          : (unsigned)kc * (unsigned)ld + (unsigned)r;
+        c.off = (r < rows) ? e * (unsigned)sizeof(T) : NG_OOB_OFFSET;
+        return c;
+    }
+
+    __device__ __forceinline__ Tile tile(int /*kt*/, int k0, int zb) const
+    {
+        Tile t;
+        t.p = base + (long)zb * ldz + (long)k0 * (LAYOUT == KC ? 1 : ld);
+        t.rsrc = make_rsrc(t.p);
+        t.krem = kdim - k0;
+        return t;
+    }
+
+    __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const
     {
         constexpr int EPC = Elem<T>::EPC;
-        const T* p = base + (long)zb * ldz;
-        uint4_t out = {0u, 0u, 0u, 0u};
         if (VEC) {
-            if (r < rows && k < kdim) {
-                const T* q = (LAYOUT == KC) ? p + (long)r * ld + k : p + (long)k * ld + r;
-                out = *reinterpret_cast<const uint4_t*>(q);
-            }
+            // rows past the matrix edge and contraction indices past kdim read as zero
+            return buffer_load_chunk(t.rsrc, (c.k < t.krem) ? c.off : NG_OOB_OFFSET);
         } else {
+            const T* p = t.p;
             T tmp[EPC];
 #pragma unroll
             for (int e = 0; e < EPC; e++) {
-                const int rr = (LAYOUT == KC) ? r : r + e;
-                const int kk = (LAYOUT == KC) ? k + e : k;
-                tmp[e] = (rr < rows && kk < kdim)
+                const int rr = (LAYOUT == KC) ? c.r : c.r + e;
+                const int kk = (LAYOUT == KC) ? c.k + e : c.k;
+                tmp[e] = (rr < rows && kk < t.krem)
                              ? ((LAYOUT == KC) ? p[(long)rr * ld + kk] : p[(long)kk * ld + rr])
                              : (T)0;
             }
-            out = *reinterpret_cast<const uint4_t*>(tmp);
+            return *reinterpret_cast<const uint4_t*>(tmp);
         }
-        return out;
     }
 };
 
@@ -192,6 +237,22 @@ __device__ __forceinline__ void tile_of_block(const CoreShape& s, int& tm, int& 
     tm = pid % s.tiles_m;
     tn = pid / s.tiles_m;
 }
+
+// Scheduling directive for one k-step.  After each MFMA: two LDS reads of the
+// next step's fragments until they are used up; one global load after every
+// other MFMA until the step's share of the next tile is issued.
+template <int I, int N_MFMA, int N_READS, int N_LOADS>
+struct InterleaveStep {
+    static __device__ __forceinline__ void emit()
+    {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+        if constexpr (2 * I < N_READS)
+            __builtin_amdgcn_sched_group_barrier(0x100, (N_READS - 2 * I) >= 2 ? 2 : 1, 0);   // LDS reads
+        if constexpr ((I & 1) == 1 && (I / 2) < N_LOADS)
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // one global load
+        if constexpr (I + 1 < N_MFMA) InterleaveStep<I + 1, N_MFMA, N_READS, N_LOADS>::emit();
+    }
+};
 
 // One 32-row band of a wavefront's accumulators: registers -> private LDS
 // staging -> 8-column chunks handed to the epilogue functor.  The band index is
@@ -243,7 +304,7 @@ void mfma_gemm_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     static_assert(TA::CHUNKS % NT == 0 && TB::CHUNKS % NT == 0, "tile chunks must divide evenly over threads");
     constexpr int TM = BM / WM / 32;
     constexpr int TN = BN / WN / 32;
-    static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % KSTEP == 0, "bad tile shape");
+    static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % (2 * KSTEP) == 0, "bad tile shape");
 
     constexpr int STAGE = TA::BYTES + TB::BYTES;
     constexpr int WTN = BN / WN;                 // columns of a wavefront's sub-tile
@@ -280,9 +341,9 @@ void mfma_gemm_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     typename ALoad::Ctx actx[CPT_A];
     typename BLoad::Ctx bctx[CPT_B];
 #pragma unroll
-    for (int i = 0; i < CPT_A; i++) actx[i] = aload.prepare(m0 + ra_r[i]);
+    for (int i = 0; i < CPT_A; i++) actx[i] = aload.prepare(m0 + ra_r[i], ra_k[i]);
 #pragma unroll
-    for (int i = 0; i < CPT_B; i++) bctx[i] = bload.prepare(n0 + rb_r[i]);
+    for (int i = 0; i < CPT_B; i++) bctx[i] = bload.prepare(n0 + rb_r[i], rb_k[i]);
 
     uint4_t ra[CPT_A], rb[CPT_B];
     float16_t acc[TM][TN];
@@ -293,13 +354,35 @@ void mfma_gemm_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    auto gload = [&](int t) {
-        const int pass = t / s.k_tiles;
-        const int k0 = (t - pass * s.k_tiles) * BK;
+    // position of the next tile to fetch: (pass, tile inside the pass), kept
+    // incrementally so that no division runs inside the loop
+    int g_pass = t_begin / s.k_tiles;
+    int g_kt = t_begin - g_pass * s.k_tiles;
+    // Global loads of the next tile are issued in NSTEP-1 parts, one inside each
+    // of the first k-steps, so that the address pipeline is fed at its own pace
+    // instead of blocking instruction issue with a burst at the top of the tile.
+    constexpr int N_CHUNKS = CPT_A + CPT_B;
+    constexpr int G_PARTS = (BK / KSTEP > 1) ? BK / KSTEP - 1 : 1;
+    constexpr int G_PER = (N_CHUNKS + G_PARTS - 1) / G_PARTS;
+    typename ALoad::Tile g_ta;
+    typename BLoad::Tile g_tb;
+    auto gtile = [&]() {
+        g_ta = aload.tile(g_kt, g_kt * BK, z + g_pass);
+        g_tb = bload.tile(g_kt, g_kt * BK, z + g_pass);
+        if (++g_kt == s.k_tiles) { g_kt = 0; g_pass++; }
+    };
+    auto gload_part = [&](int part) {
 #pragma unroll
-        for (int i = 0; i < CPT_A; i++) ra[i] = aload.load(actx[i], k0 + ra_k[i], z + pass);
+        for (int c = 0; c < N_CHUNKS; c++) {
+            if (c / G_PER != part) continue;
+            if (c < CPT_A) ra[c < CPT_A ? c : 0] = aload.load(g_ta, actx[c < CPT_A ? c : 0]);
+            else           rb[c >= CPT_A ? c - CPT_A : 0] = bload.load(g_tb, bctx[c >= CPT_A ? c - CPT_A : 0]);
+        }
+    };
+    auto gload = [&]() {
+        gtile();
 #pragma unroll
-        for (int i = 0; i < CPT_B; i++) rb[i] = bload.load(bctx[i], k0 + rb_k[i], z + pass);
+        for (int part = 0; part < G_PARTS; part++) gload_part(part);
     };
     auto sstore = [&](int buf) {
 #pragma unroll
@@ -308,36 +391,82 @@ void mfma_gemm_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
         for (int i = 0; i < CPT_B; i++) *reinterpret_cast<uint4_t*>(smem + buf * STAGE + TA::BYTES + rb_off[i]) = rb[i];
     };
 
+    // Main loop, software pipelined for one wavefront per SIMD:
+    //  * global loads of tile t+1 are issued at the top of tile t and land in
+    //    registers while tile t is multiplied;
+    //  * MFMA fragments are double buffered: the LDS reads of k-step s+1 are
+    //    issued before the MFMAs of step s;
+    //  * the registers of tile t+1 are written to the other LDS stage and the
+    //    single barrier of the iteration is taken BEFORE the last k-step, so the
+    //    first fragments of tile t+1 are already in flight while the last MFMAs
+    //    of tile t execute.
+    constexpr int NSTEP = BK / KSTEP;
+    Frag<T> fa[2][TM], fb[2][TN];
+
+    auto load_frags = [&](int stage_buf, int step, Frag<T> (&a)[TM], Frag<T> (&b)[TN]) {
+        const char* a_lds = smem + stage_buf * STAGE;
+        const char* b_lds = a_lds + TA::BYTES;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+            a[i] = FragLoader<T, LA, TA::PITCH>::load(a_lds, wm * (BM / WM) + i * 32, step * KSTEP, lane);
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+            b[j] = FragLoader<T, LB, TB::PITCH>::load(b_lds, wn * (BN / WN) + j * 32, step * KSTEP, lane);
+    };
+    auto multiply = [&](const Frag<T> (&a)[TM], const Frag<T> (&b)[TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) mfma_step(a[i], b[j], acc[i][j]);
+    };
+
     if (t_begin < t_end) {
-        gload(t_begin);
+        gload();
         sstore(0);
     }
     __syncthreads();
+    if (t_begin < t_end) load_frags(0, 0, fa[0], fb[0]);
 
-    for (int t = t_begin; t < t_end; t++) {
+    // LDS read instructions one k-step issues for the next step's fragments
+    constexpr bool IS_HALF = (sizeof(T) == 2);
+    constexpr int RD_A = (LA == KC) ? 1 : (IS_HALF ? 2 : 4);
+    constexpr int RD_B = (LB == KC) ? 1 : (IS_HALF ? 2 : 4);
+    constexpr int N_READS = TM * RD_A + TN * RD_B;
+    constexpr int N_MFMA = TM * TN * (IS_HALF ? 1 : 4);
+
+    // One k-step: prefetch the next fragments, multiply the current ones, and
+    // tell the scheduler to issue the prefetch reads at the head of the step,
+    // two after each MFMA, instead of sinking them next to their first use.
+    auto step = [&](int rd_buf, int rd_step, Frag<T> (&na)[TM], Frag<T> (&nb)[TN],
+                    const Frag<T> (&ca)[TM], const Frag<T> (&cb)[TN], int load_part) {
+        if (load_part >= 0) gload_part(load_part);
+        load_frags(rd_buf, rd_step, na, nb);
+        multiply(ca, cb);
+        if (load_part >= 0) InterleaveStep<0, N_MFMA, N_READS, G_PER>::emit();
+        else                InterleaveStep<0, N_MFMA, N_READS, 0>::emit();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // every tile but the last: one straight-line block per iteration
+    for (int t = t_begin; t + 1 < t_end; t++) {
         const int buf = (t - t_begin) & 1;
-        const bool more = (t + 1 < t_end);
-        if (more) gload(t + 1);
-
-        const char* a_lds = smem + buf * STAGE;
-        const char* b_lds = a_lds + TA::BYTES;
+        gtile();
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int kk = 0; kk < BK; kk += KSTEP) {
-            Frag<T> fa[TM], fb[TN];
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-                fa[i] = FragLoader<T, LA, TA::PITCH>::load(a_lds, wm * (BM / WM) + i * 32, kk, lane);
-#pragma unroll
-            for (int j = 0; j < TN; j++)
-                fb[j] = FragLoader<T, LB, TB::PITCH>::load(b_lds, wn * (BN / WN) + j * 32, kk, lane);
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++) mfma_step(fa[i], fb[j], acc[i][j]);
-        }
-
-        if (more) sstore(buf ^ 1);
+        for (int s = 0; s < NSTEP - 1; s++)
+            step(buf, s + 1, fa[(s + 1) & 1], fb[(s + 1) & 1], fa[s & 1], fb[s & 1], s);
+        sstore(buf ^ 1);
         __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        step(buf ^ 1, 0, fa[NSTEP & 1], fb[NSTEP & 1], fa[(NSTEP - 1) & 1], fb[(NSTEP - 1) & 1], -1);
+    }
+    // last tile: nothing left to fetch
+    if (t_begin < t_end) {
+        const int buf = (t_end - 1 - t_begin) & 1;
+#pragma unroll
+        for (int s = 0; s < NSTEP - 1; s++)
+            step(buf, s + 1, fa[(s + 1) & 1], fb[(s + 1) & 1], fa[s & 1], fb[s & 1], -1);
+        multiply(fa[(NSTEP - 1) & 1], fb[(NSTEP - 1) & 1]);
     }
 
     // Epilogue.  The 32x32 MFMA block leaves lane l with column (l & 31) and rows
@@ -406,9 +535,19 @@ struct ScaleStoreEpilogue {
     __device__ __forceinline__ void store8(int i, int j0, int z, int /*split*/, const float (&acc)[8]) const
     {
         if (i >= m || j0 >= n) return;
-        if (vec) {
-            constexpr int NV = (int)sizeof(bits_t) * 8 / 16;   // 16-byte pieces per 8 elements
-            bits_t* p = reinterpret_cast<bits_t*>(C + (long)z * ldcz + (long)i * ldc + j0);
+        constexpr int NV = (int)sizeof(bits_t) * 8 / 16;   // 16-byte pieces per 8 elements
+        bits_t* p = reinterpret_cast<bits_t*>(C + (long)z * ldcz + (long)i * ldc + j0);
+        if (vec && beta == 0.0f && sr_bits == 0) {
+            // common case, kept free of the rounding-stream arithmetic:
+            // scale, optional relu, nearest rounding, 16-byte stores
+            const float lo = relu ? 0.0f : -3.402823466e+38f;
+            bits_t out[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) out[e] = StoreBits<T>::round(fmaxf(acc[e] * alpha, lo), 0, 0, 0, 0);
+#pragma unroll
+            for (int q = 0; q < NV; q++)
+                reinterpret_cast<uint4_t*>(p)[q] = reinterpret_cast<const uint4_t*>(out)[q];
+        } else if (vec) {
             bits_t out[8];
             if (beta != 0.0f) {
 #pragma unroll
