@@ -489,7 +489,7 @@ template <> struct StoreBits<_Float16> {
     typedef unsigned short bits_t;
     static __device__ __forceinline__ bits_t round(float v, unsigned sr_bits, unsigned seed, unsigned stream, unsigned idx)
     {
-        return sr_bits ? ng_sr_f16(v, sr_bits, ng_rand32(seed, stream, idx)) : ng_f32_to_f16_rn(v);
+        return sr_bits ? ng_sr_f16(v, sr_bits, ng_rand_sr16(seed, stream, idx)) : ng_f32_to_f16_rn(v);
     }
     static __device__ __forceinline__ float widen(bits_t b) { return ng_f16_to_f32(b); }
 };

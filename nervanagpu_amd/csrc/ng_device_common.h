@@ -21,12 +21,29 @@ NG_DEV unsigned ng_fmix32(unsigned h)
     return h;
 }
 
-// 32 random bits for element idx of launch `stream` under `seed`.
+// 32 random bits for element idx of launch `stream` under `seed`.  The two keys
+// depend only on (seed, stream) and are wavefront-uniform (scalar unit); per
+// element the cost is two 32-bit multiplies and a few shifts/xors.  For fixed
+// keys the map idx -> bits is a bijection.
 NG_DEV unsigned ng_rand32(unsigned seed, unsigned stream, unsigned idx)
 {
-    unsigned h = ng_fmix32(idx + seed * 0x9E3779B1u);
-    unsigned k = stream * 0x85EBCA77u + 0xC2B2AE3Du;
-    return ng_fmix32(h ^ k);
+    const unsigned ka = ng_fmix32(seed ^ 0x9E3779B9u) + stream * 0x85EBCA77u;
+    const unsigned kb = ng_fmix32(stream + 0xC2B2AE3Du) ^ seed;
+    unsigned x = idx + ka;
+    x ^= x >> 16; x *= 0x7FEB352Du;
+    x ^= kb;
+    x ^= x >> 15; x *= 0x846CA68Bu;
+    x ^= x >> 16;
+    return x;
+}
+
+// Random word for the fp16 stochastic rounding of element idx: fp16 needs at
+// most 16 random bits, so elements 2i and 2i+1 share the draw of index i; the
+// even element uses its high half, the odd one its low half.
+NG_DEV unsigned ng_rand_sr16(unsigned seed, unsigned stream, unsigned idx)
+{
+    const unsigned h = ng_rand32(seed, stream, idx >> 1);
+    return (idx & 1u) ? (h << 16) : h;
 }
 
 // uniform in [0,1]: nearest-even convert of 32 bits, times 2^-32
@@ -51,27 +68,27 @@ NG_DEV float ng_sr_f32(float v, unsigned bits, unsigned r)
 }
 
 // fp32 -> fp16 bits, round toward zero (overflow saturates at 65504,
-// subnormal results are truncated).
+// subnormal results are truncated): the hardware pack-convert does exactly this.
 NG_DEV unsigned short ng_f32_to_f16_rz(float v)
 {
-    unsigned u    = __float_as_uint(v);
-    unsigned sign = (u >> 16) & 0x8000u;
-    unsigned mag  = u & 0x7FFFFFFFu;
-    int      e    = (int)(mag >> 23);
-    unsigned man  = mag & 0x7FFFFFu;
-    unsigned h;
-    if (mag > 0x7F800000u)       h = 0x7E00u;
-    else if (mag == 0x7F800000u) h = 0x7C00u;
-    else if (mag >= 0x47800000u) h = 0x7BFFu;
-    else if (e >= 113)           h = ((unsigned)(e - 112) << 10) | (man >> 13);
-    else if (e < 102)            h = 0u;
-    else                         h = (man | 0x800000u) >> (unsigned)(126 - e);
-    return (unsigned short)(h | sign);
+    typedef _Float16 ng_half2_t __attribute__((ext_vector_type(2)));
+    const ng_half2_t h = __builtin_bit_cast(ng_half2_t, __builtin_amdgcn_cvt_pkrtz(v, 0.0f));
+    const _Float16 lo = h[0];
+    return __builtin_bit_cast(unsigned short, lo);
 }
 
+// fp32 -> fp16 bits with stochastic rounding at `bits` (1..10) mantissa bits.
+// Finite magnitudes are first clamped to the largest fp16 value, so the random
+// increment can never carry into the infinity pattern; the final truncating
+// convert then drops whatever lies below the fp16 grid.
 NG_DEV unsigned short ng_sr_f16(float v, unsigned bits, unsigned r)
 {
-    return ng_f32_to_f16_rz(ng_sr_f32(v, bits, r));
+    const unsigned u    = __float_as_uint(v);
+    const unsigned d    = 23u - bits;
+    const unsigned mag  = u & 0x7FFFFFFFu;
+    unsigned m2 = (min(mag, 0x477FE000u) + (r >> (32u - d))) & (0xFFFFFFFFu << d);
+    m2 = (mag >= 0x7F800000u) ? mag : m2;
+    return ng_f32_to_f16_rz(__uint_as_float((u & 0x80000000u) | m2));
 }
 
 // nearest-even fp32 -> fp16 bits

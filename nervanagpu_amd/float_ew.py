@@ -82,6 +82,7 @@ _ew_types = {
 
 MAX_CACHED_PER_LANE = 32     # fp32 registers per operand kept resident per lane
 MAX_THREADS = 1024
+FLAT_UNROLL = 4              # independent vectors per lane per pass of the flat kernel
 
 
 def _contiguous_strides(shape):
@@ -268,7 +269,7 @@ class _Emitter(object):
 class KernelSpec(object):
     """Everything that selects a generated kernel (hashable via .key)."""
 
-    def __init__(self, type_args, tensors, mode, vec, threads, items, n_onehot):
+    def __init__(self, type_args, tensors, mode, vec, threads, items, n_onehot, rng_pair=False):
         # tensors: list of (arg_id, dtype_code, access, take_axis, is_out)
         #   access: 'vec' contiguous+aligned along the row, 'strided', 'row' (one value per row)
         self.type_args = tuple(type_args)
@@ -278,7 +279,10 @@ class KernelSpec(object):
         self.threads = threads
         self.items = items            # >0: row cached in registers with this many vectors per lane; 0: streaming
         self.n_onehot = n_onehot
-        self.key = (self.type_args, self.tensors, mode, vec, threads, items, n_onehot)
+        # rng_pair: vector stores start at an even random-stream index with unit
+        # stride, so fp16 stochastic stores can share one draw per element pair
+        self.rng_pair = bool(rng_pair)
+        self.key = (self.type_args, self.tensors, mode, vec, threads, items, n_onehot, self.rng_pair)
         self._tensor_by_id = dict((t[0], t) for t in tensors)
 
     def tensor_value(self, arg_id, item, v):
@@ -314,8 +318,9 @@ def _gen_load(spec, t, item, base_col, out, indent, bound="n"):
         out.append("%s    x%d_%s[v] = (%s + v < %s) ? (float)p%d[%s] : 0.0f;" % (pad, arg_id, item, base_col, bound, arg_id, idx))
 
 
-def _gen_round(code, value, rounding, idx):
-    """expression of storage type for fp32 `value`"""
+def _gen_round(code, value, rounding, idx, rword=None):
+    """expression of storage type for fp32 `value`; `rword` overrides the
+    random word of an fp16 stochastic store (shared pair draws)"""
     ct, rng = _ew_types[code]
     if code == "f4":
         if rounding:
@@ -323,7 +328,9 @@ def _gen_round(code, value, rounding, idx):
         return value
     if code == "f2":
         if rounding:
-            return "__builtin_bit_cast(_Float16, ng_sr_f16(%s, sr_bits, ng_rand32(rng_seed, rng_stream, %s)))" % (value, idx)
+            if rword is None:
+                rword = "ng_rand_sr16(rng_seed, rng_stream, %s)" % idx
+            return "__builtin_bit_cast(_Float16, ng_sr_f16(%s, sr_bits, %s))" % (value, rword)
         return "(_Float16)(%s)" % value
     return "(%s)ng_rint_sat(%s, %rf, %rf)" % (ct, value, rng[0], rng[1])
 
@@ -374,6 +381,14 @@ def generate_source(spec, name="ew_kernel"):
     L.append("extern \"C\" __global__ __launch_bounds__(THREADS) void %s(\n    %s)\n{" % (name, ",\n    ".join(decl)))
     L.append("    const int tid = threadIdx.x;")
 
+    def pair_words(o, pad, code):
+        """shared draws for a vector of fp16 stochastic stores"""
+        if not (spec.rng_pair and rounding and code == "f2"):
+            return [None] * V
+        for k in range(V // 2):
+            o.append("%sconst unsigned rh%d_ = ng_rand32(rng_seed, rng_stream, (rng_idx >> 1) + %du);" % (pad, k, k))
+        return ["rh%d_" % (v // 2) if v % 2 == 0 else "(rh%d_ << 16)" % (v // 2) for v in range(V)]
+
     def store_code(item, base_col, vals, indent):
         pad = " " * indent
         arg_id, code, access, take_axis, _ = out_t
@@ -381,8 +396,9 @@ def generate_source(spec, name="ew_kernel"):
         o = []
         if access == "vec" and V > 1:
             o.append("%s{ typedef %s vt_ __attribute__((ext_vector_type(%d))); vt_ o_;" % (pad, ct, V))
+            rwords = pair_words(o, pad + "  ", code)
             for v in range(V):
-                o.append("%s  o_[%d] = %s;" % (pad, v, _gen_round(code, vals[v], rounding, "rng_idx + %du" % v if not rng_strided else "rng_idx + %du * rng_cm" % v)))
+                o.append("%s  o_[%d] = %s;" % (pad, v, _gen_round(code, vals[v], rounding, "rng_idx + %du" % v if not rng_strided else "rng_idx + %du * rng_cm" % v, rwords[v])))
             o.append("%s  *reinterpret_cast<vt_*>(p%d + (long)(%s)) = o_; }" % (pad, arg_id, base_col))
         else:
             for v in range(V):
@@ -399,9 +415,11 @@ def generate_source(spec, name="ew_kernel"):
 
     if flat:
         rng_strided = False
-        # one flat grid-stride loop over vectors of VEC consecutive elements
+        # each workgroup walks chunks of FLAT_UNROLL * THREADS vectors; inside a
+        # full chunk the per-vector bodies are independent, so their loads issue
+        # back to back before the first use
         L.append("    const long nvec = rows;   // number of VEC-wide vectors")
-        L.append("    for (long g = (long)blockIdx.x * THREADS + tid; g < nvec; g += (long)gridDim.x * THREADS) {")
+        L.append("    auto vec_body = [&](const long g) {")
         L.append("        const long col = g * VEC;")
         L.append("        const unsigned rng_idx = (unsigned)col;")
         body = []
@@ -429,11 +447,20 @@ def generate_source(spec, name="ew_kernel"):
         ct = _ctype(code)
         if V > 1:
             L.append("        { typedef %s vt_ __attribute__((ext_vector_type(%d))); vt_ o_;" % (ct, V))
+            rwords = pair_words(L, "          ", code)
             for v in range(V):
-                L.append("          o_[%d] = %s;" % (v, _gen_round(code, vals[v], rounding, "rng_idx + %du" % v)))
+                L.append("          o_[%d] = %s;" % (v, _gen_round(code, vals[v], rounding, "rng_idx + %du" % v, rwords[v])))
             L.append("          *reinterpret_cast<vt_*>(p%d + col) = o_; }" % arg_id)
         else:
             L.append("        p%d[col] = %s;" % (arg_id, _gen_round(code, vals[0], rounding, "rng_idx")))
+        L.append("    };")
+        L.append("    const long chunk = (long)THREADS * %d;" % FLAT_UNROLL)
+        L.append("    for (long base = (long)blockIdx.x * chunk; base < nvec; base += (long)gridDim.x * chunk) {")
+        L.append("        if (base + chunk <= nvec) {")
+        L.append("            _Pragma(\"unroll\") for (int u = 0; u < %d; u++) vec_body(base + (long)u * THREADS + tid);" % FLAT_UNROLL)
+        L.append("        } else {")
+        L.append("            for (long g = base + tid; g < nvec; g += THREADS) vec_body(g);")
+        L.append("        }")
         L.append("    }")
         L.append("}")
         return "\n".join(L), args
@@ -850,7 +877,8 @@ def analyse(args):
         plan.rows = size // vec
         plan.threads = 256
         plan.items = 0
-        plan.grid = max(1, min((plan.rows + 255) // 256, 8192))
+        per_block = 256 * FLAT_UNROLL
+        plan.grid = max(1, min((plan.rows + per_block - 1) // per_block, 16384))
         plan.rng_rm, plan.rng_cm = 0, 1
         tensors = [(i, v["dtype"], "vec", 0, v["is_out"]) for i, v in sorted(values.items()) if "ptr" in v]
     else:
@@ -913,7 +941,8 @@ def analyse(args):
                 access = "strided"
             tensors.append((i, v["dtype"], access, v["take_axis"], v["is_out"]))
 
-    plan.spec = KernelSpec(type_args, tensors, plan.mode, plan.vec, plan.threads, plan.items, len(onehots))
+    rng_pair = plan.vec > 1 and plan.rng_cm == 1 and plan.rng_rm % 2 == 0
+    plan.spec = KernelSpec(type_args, tensors, plan.mode, plan.vec, plan.threads, plan.items, len(onehots), rng_pair)
     return plan
 
 

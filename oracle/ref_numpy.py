@@ -34,7 +34,7 @@ import numpy as np
 
 __all__ = [
     "contiguous_strides", "magic32", "fast_ew_dims", "gemm_tile_heuristic",
-    "rand32", "rand_uniform", "f32_to_f16_rz", "round_fp16_rn", "round_int",
+    "rand32", "rand_sr16", "rand_uniform", "f32_to_f16_rz", "round_fp16_rn", "round_int",
     "round_stochastic_fp16", "round_stochastic_fp32", "round_store",
     "ref_dot", "ref_batched_dot",
     "conv_out_dims", "conv_pixel_indices", "ref_conv_fprop", "ref_conv_bprop",
@@ -131,27 +131,43 @@ def gemm_tile_heuristic(op, m, n, sm_count):
 _U32 = np.uint32
 
 
-def _fmix32(h):
-    h = h.astype(np.uint32, copy=True)
-    h ^= h >> _U32(16)
-    h *= _U32(0x85EBCA6B)
-    h ^= h >> _U32(13)
-    h *= _U32(0xC2B2AE35)
-    h ^= h >> _U32(16)
+def _fmix32_scalar(h):
+    h &= 0xFFFFFFFF
+    h ^= h >> 16
+    h = (h * 0x85EBCA6B) & 0xFFFFFFFF
+    h ^= h >> 13
+    h = (h * 0xC2B2AE35) & 0xFFFFFFFF
+    h ^= h >> 16
     return h
 
 
 def rand32(seed, stream, idx):
     """32 random bits for element `idx` of launch `stream` under `seed`.
-    Two rounds of the murmur3 finaliser; a bijection of idx for fixed
-    (seed, stream), so a full sweep of idx is exactly uniform."""
+    Two keys derived from (seed, stream) with the murmur3 finaliser, then a
+    two-multiply integer hash of idx; a bijection of idx for fixed keys, so a
+    full sweep of idx is exactly uniform."""
+    seed = int(seed) & 0xFFFFFFFF
+    stream = int(stream) & 0xFFFFFFFF
+    ka = (_fmix32_scalar(seed ^ 0x9E3779B9) + stream * 0x85EBCA77) & 0xFFFFFFFF
+    kb = _fmix32_scalar((stream + 0xC2B2AE3D) & 0xFFFFFFFF) ^ seed
     with np.errstate(over="ignore"):
-        idx = np.asarray(idx).astype(np.uint32)
-        seed = _U32(int(seed) & 0xFFFFFFFF)
-        stream = _U32(int(stream) & 0xFFFFFFFF)
-        h = _fmix32(idx + seed * _U32(0x9E3779B1))
-        k = stream * _U32(0x85EBCA77) + _U32(0xC2B2AE3D)
-        return _fmix32(h ^ k)
+        x = np.asarray(idx).astype(np.uint32) + _U32(ka)
+        x ^= x >> _U32(16)
+        x *= _U32(0x7FEB352D)
+        x ^= _U32(kb)
+        x ^= x >> _U32(15)
+        x *= _U32(0x846CA68B)
+        x ^= x >> _U32(16)
+    return x
+
+
+def rand_sr16(seed, stream, idx):
+    """Random word for the fp16 stochastic rounding of element `idx`: elements
+    2i and 2i+1 share the draw of index i (fp16 needs at most 16 random bits);
+    the even element uses the high half, the odd one the low half."""
+    idx = np.asarray(idx).astype(np.uint32)
+    h = rand32(seed, stream, idx >> _U32(1))
+    return np.where((idx & _U32(1)) != 0, h << _U32(16), h).astype(np.uint32)
 
 
 def rand_uniform(seed, stream, idx):
@@ -198,7 +214,7 @@ def round_int(x, dtype):
     return np.clip(r, info.min, info.max).astype(dtype)
 
 
-def _sr_bits(x, bits, r):
+def _sr_bits(x, bits, r, clamp_mag=None):
     u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
     r = np.asarray(r).astype(np.uint32)
     d = 23 - int(bits)
@@ -207,8 +223,9 @@ def _sr_bits(x, bits, r):
     sign = u & _U32(0x80000000)
     mag = u & _U32(0x7FFFFFFF)
     finite = mag < _U32(0x7F800000)
+    base = mag if clamp_mag is None else np.minimum(mag, _U32(clamp_mag))
     with np.errstate(over="ignore"):
-        m2 = (mag + (r >> _U32(32 - d))) & mask
+        m2 = (base + (r >> _U32(32 - d))) & mask
     m2 = np.where(m2 >= _U32(0x7F800000), _U32(0x7F7FFFFF) & mask, m2)
     m2 = np.where(finite, m2, mag)
     return (sign | m2).astype(np.uint32)
@@ -224,7 +241,9 @@ def round_stochastic_fp32(x, bits, r):
 def round_stochastic_fp16(x, bits, r):
     """fp32 -> fp16 (returned as float16) with stochastic rounding at `bits`
     (<=10) mantissa bits (fp32_to_fp16_rand, nervanagpu/float_ew.py:182-201)."""
-    v = _sr_bits(x, min(int(bits), 10), r).view(np.float32)
+    # finite magnitudes saturate at the largest fp16 value (65504 = 0x477FE000)
+    # before the random increment, so it can never carry into infinity
+    v = _sr_bits(x, min(int(bits), 10), r, clamp_mag=0x477FE000).view(np.float32)
     return f32_to_f16_rz(v).view(np.float16)
 
 

@@ -6,6 +6,7 @@ import os
 
 
 def fmix(h):
+    h &= 0xFFFFFFFF
     h ^= h >> 16
     h = (h * 0x85EBCA6B) & 0xFFFFFFFF
     h ^= h >> 13
@@ -15,9 +16,16 @@ def fmix(h):
 
 
 def r32(seed, stream, idx):
-    h = fmix((idx + seed * 0x9E3779B1) & 0xFFFFFFFF)
-    k = (stream * 0x85EBCA77 + 0xC2B2AE3D) & 0xFFFFFFFF
-    return fmix(h ^ k)
+    ka = (fmix(seed ^ 0x9E3779B9) + stream * 0x85EBCA77) & 0xFFFFFFFF
+    kb = fmix((stream + 0xC2B2AE3D) & 0xFFFFFFFF) ^ seed
+    x = (idx + ka) & 0xFFFFFFFF
+    x ^= x >> 16
+    x = (x * 0x7FEB352D) & 0xFFFFFFFF
+    x ^= kb
+    x ^= x >> 15
+    x = (x * 0x846CA68B) & 0xFFFFFFFF
+    x ^= x >> 16
+    return x
 
 
 if __name__ == "__main__":

@@ -278,13 +278,13 @@ def test_stochastic_rounding_store_bit_exact(ng):
     from nervanagpu_amd import NervanaGPU
     ngs = NervanaGPU(stochastic_round=True, seed=77)
     rng = np.random.default_rng(7)
-    for shape in ((64, 1024), (33, 250)):
+    for shape in ((64, 1024), (33, 250), (33, 251)):
         a = (rng.standard_normal(shape) * 3).astype(np.float32)
         A = ngs.array(a, dtype=np.float32)
         H = ngs.empty(shape)                # fp16, rounding=10
         assert H.rounding == 10
         H[:] = A                            # plain contiguous copy-convert
-        r = orc.rand32(77, ngs.rng_counter, np.arange(a.size, dtype=np.uint32)).reshape(shape)
+        r = orc.rand_sr16(77, ngs.rng_counter, np.arange(a.size, dtype=np.uint32)).reshape(shape)
         assert np.array_equal(H.get().view(np.uint16), orc.round_stochastic_fp16(a, 10, r).view(np.uint16))
         # row-mode kernel (reduction + broadcast) with SR store: take the kernel's own
         # fp32 values from a second, unrounded run of the same expression
@@ -292,13 +292,13 @@ def test_stochastic_rounding_store_bit_exact(ng):
         P.rounding = 0
         P[:] = bn_expr(ngs, A, 1e-3)
         H[:] = bn_expr(ngs, A, 1e-3)
-        r = orc.rand32(77, ngs.rng_counter, np.arange(a.size, dtype=np.uint32)).reshape(shape)
+        r = orc.rand_sr16(77, ngs.rng_counter, np.arange(a.size, dtype=np.uint32)).reshape(shape)
         assert np.array_equal(H.get().view(np.uint16), orc.round_stochastic_fp16(P.get(), 10, r).view(np.uint16))
         # fewer bits, transposed output walk (axis 0 reduction)
         H.rounding = 4
         H[:] = A - ng_mean0(ngs, A)
         P[:] = A - ng_mean0(ngs, A)
-        r = orc.rand32(77, ngs.rng_counter, np.arange(a.size, dtype=np.uint32)).reshape(shape)
+        r = orc.rand_sr16(77, ngs.rng_counter, np.arange(a.size, dtype=np.uint32)).reshape(shape)
         assert np.array_equal(H.get().view(np.uint16), orc.round_stochastic_fp16(P.get(), 4, r).view(np.uint16))
         H.rounding = 10
     # fp32 SR
@@ -313,7 +313,7 @@ def test_stochastic_rounding_store_bit_exact(ng):
                   dtype=np.float32)
     S = ngs.empty(sp.shape)
     S[:] = ngs.array(sp, dtype=np.float32)
-    r = orc.rand32(77, ngs.rng_counter, np.arange(sp.size, dtype=np.uint32)).reshape(sp.shape)
+    r = orc.rand_sr16(77, ngs.rng_counter, np.arange(sp.size, dtype=np.uint32)).reshape(sp.shape)
     assert np.array_equal(S.get().view(np.uint16), orc.round_stochastic_fp16(sp, 10, r).view(np.uint16))
 
 

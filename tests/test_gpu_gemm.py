@@ -213,7 +213,7 @@ def test_stochastic_rounding_bit_exact(ng):
         stream = ngs.rng_counter
         pre = orc.ref_dot(A, B, relu=True)                      # exact in fp32
         assert np.array_equal(pre.astype(np.float64), np.maximum(A.astype(np.float64) @ B.astype(np.float64), 0))
-        r = orc.rand32(1234, stream, np.arange(m * n, dtype=np.uint32)).reshape(m, n)
+        r = orc.rand_sr16(1234, stream, np.arange(m * n, dtype=np.uint32)).reshape(m, n)
         exp = orc.round_stochastic_fp16(pre, 10, r)
         got = C.get()
         assert np.array_equal(got.view(np.uint16), exp.view(np.uint16)), op
