@@ -25,6 +25,8 @@
 
 #include "gemm_core.h"
 
+#include <type_traits>
+
 namespace ng {
 
 // a tap (or, in flat tables, one contraction row): element offset relative to
@@ -122,6 +124,9 @@ struct GatherColsLoader {
     FastDiv         blk_div;    // BLOCKED: tile index -> tap (blocks per tap = nblk)
     int             nblk;
 
+    // same-type inputs are plain 16-byte buffer loads (see DenseLoader::DIRECT)
+    static constexpr bool DIRECT = std::is_same<T, TIN>::value;
+
     struct Ctx { int base, z0, y0, x0, kr; };
     struct Tile { BufferRsrc rsrc; int toff, dz, dy, dx, k0; };
 
@@ -156,20 +161,26 @@ struct GatherColsLoader {
         return t;
     }
 
-    __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const
+    // byte offset of the chunk, out of range for taps outside the image
+    __device__ __forceinline__ unsigned offset(const Tile& t, const Ctx& c) const
     {
         constexpr int ES = ChunkFetch<T, TIN>::ES;
         if (BLOCKED) {
             const bool ok = (unsigned)(c.z0 + t.dz) < (unsigned)lim_d && (unsigned)(c.y0 + t.dy) < (unsigned)lim_h &&
                             (unsigned)(c.x0 + t.dx) < (unsigned)lim_w;
-            return ChunkFetch<T, TIN>::get(t.rsrc, ok ? (unsigned)(c.base + t.toff) * ES : NG_OOB_OFFSET);
+            return ok ? (unsigned)(c.base + t.toff) * ES : NG_OOB_OFFSET;
         } else {
             const int k = t.k0 + c.kr;
             const TapEntry e = tab[min(k, J - 1)];
             const bool ok = k < J && (unsigned)(c.z0 + e.dz) < (unsigned)lim_d &&
                             (unsigned)(c.y0 + e.dy) < (unsigned)lim_h && (unsigned)(c.x0 + e.dx) < (unsigned)lim_w;
-            return ChunkFetch<T, TIN>::get(t.rsrc, ok ? (unsigned)(c.base + e.off) * ES : NG_OOB_OFFSET);
+            return ok ? (unsigned)(c.base + e.off) * ES : NG_OOB_OFFSET;
         }
+    }
+
+    __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const
+    {
+        return ChunkFetch<T, TIN>::get(t.rsrc, offset(t, c));
     }
 };
 
@@ -183,6 +194,8 @@ struct FilterBlockLoader {
     int      RSTK;       // elements between consecutive channels
     FastDiv  blk_div;
     int      nblk;
+
+    static constexpr bool DIRECT = true;
 
     struct Ctx { unsigned off; };
     struct Tile { BufferRsrc rsrc; };
@@ -201,6 +214,7 @@ struct FilterBlockLoader {
         t.rsrc = make_rsrc(F + (long)blk * BK * RSTK + (long)tap * K);
         return t;
     }
+    __device__ __forceinline__ unsigned offset(const Tile& /*t*/, const Ctx& c) const { return c.off; }
     __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const { return buffer_load_chunk(t.rsrc, c.off); }
 };
 
@@ -218,6 +232,8 @@ struct GatherRowsLoader {
     int             D, H, W;
     FastDiv         npt_div, pq_div, q_div;   // tiles per pixel, P*Q, Q
     int             npt;
+
+    static constexpr bool DIRECT = std::is_same<T, TIN>::value;
 
     struct Ctx { int off, dz, dy, dx, kc; };
     struct Tile { BufferRsrc rsrc; int pixbase, z0, y0, x0, k0; };
@@ -255,13 +271,13 @@ struct GatherRowsLoader {
         return t;
     }
 
-    __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const
+    __device__ __forceinline__ unsigned offset(const Tile& t, const Ctx& c) const
     {
         constexpr int ES = ChunkFetch<T, TIN>::ES;
         if (BLOCKED) {
             const bool ok = (unsigned)(t.z0 + c.dz) < (unsigned)D && (unsigned)(t.y0 + c.dy) < (unsigned)H &&
                             (unsigned)(t.x0 + c.dx) < (unsigned)W;
-            return ChunkFetch<T, TIN>::get(t.rsrc, ok ? (unsigned)(t.pixbase + c.off) * ES : NG_OOB_OFFSET);
+            return ok ? (unsigned)(t.pixbase + c.off) * ES : NG_OOB_OFFSET;
         } else {
             const int kk = t.k0 + c.kc;
             const int kc2 = min(kk, kdim - 1);
@@ -271,9 +287,13 @@ struct GatherRowsLoader {
             const int z0 = m * str_d, y0 = p * str_h, x0 = q * str_w;
             const bool ok = kk < kdim && (unsigned)(z0 + c.dz) < (unsigned)D && (unsigned)(y0 + c.dy) < (unsigned)H &&
                             (unsigned)(x0 + c.dx) < (unsigned)W;
-            return ChunkFetch<T, TIN>::get(
-                t.rsrc, ok ? (unsigned)(((z0 * H + y0) * W + x0) * N + nn + c.off) * ES : NG_OOB_OFFSET);
+            return ok ? (unsigned)(((z0 * H + y0) * W + x0) * N + nn + c.off) * ES : NG_OOB_OFFSET;
         }
+    }
+
+    __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const
+    {
+        return ChunkFetch<T, TIN>::get(t.rsrc, offset(t, c));
     }
 };
 

@@ -75,8 +75,7 @@ inline int launch_core(const AL& al, const BL& bl, const Epi& epi, int rows, int
     s.passes = 1; s.splits = splits;
     s.tiles_m = cdiv(rows, BM);
     s.tiles_n = cdiv(ncols, BN);
-    hipLaunchKernelGGL((mfma_gemm_kernel<T, BM, BN, BK, WM, WN, LA, LB, AL, BL, Epi>),
-                       dim3(s.tiles_m * s.tiles_n, splits, 1), dim3(WM * WN * 64), 0, stream, al, bl, epi, s);
+    launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB>(dim3(s.tiles_m * s.tiles_n, splits, 1), stream, al, bl, epi, s);
     NG_CHECK_LAUNCH(what);
     return 0;
 }

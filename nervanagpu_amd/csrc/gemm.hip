@@ -59,17 +59,12 @@ static int launch_gemm(const GemmArgs& g, unsigned sr_bits)
                               (((uintptr_t)g.C & 15) == 0 && g.ldc % 8 == 0 && g.ldcz % 8 == 0 && g.n % 8 == 0) ? 1u : 0u};
 
     dim3 grid(s.tiles_m * s.tiles_n, s.splits, zcount);
-    dim3 block(WM * WN * 64);
     if (s.splits == 1) {
-        hipLaunchKernelGGL((mfma_gemm_kernel<T, BM, BN, BK, WM, WN, LA, LB, DenseLoader<T, LA, VEC>,
-                                             DenseLoader<T, LB, VEC>, ScaleStoreEpilogue<T>>),
-                           grid, block, 0, g.stream, al, bl, epi, s);
+        launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB>(grid, g.stream, al, bl, epi, s);
         NG_CHECK_LAUNCH("gemm kernel");
     } else {
         PartialEpilogue pe{(float*)g.ws, g.m, g.n, zcount, (g.n % 8 == 0) ? 1u : 0u};
-        hipLaunchKernelGGL((mfma_gemm_kernel<T, BM, BN, BK, WM, WN, LA, LB, DenseLoader<T, LA, VEC>,
-                                             DenseLoader<T, LB, VEC>, PartialEpilogue>),
-                           grid, block, 0, g.stream, al, bl, pe, s);
+        launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB>(grid, g.stream, al, bl, pe, s);
         NG_CHECK_LAUNCH("gemm split kernel");
         const long total = (long)zcount * g.m * g.n;
         const int blocks = (int)std::min<long>((total + 255) / 256, 8192);

@@ -181,6 +181,10 @@ struct DenseLoader {
     int      rows;   // extent along r
     int      kdim;   // extent along k (per pass)
 
+    // a chunk is one 16-byte buffer load whose offset offset() returns, so the
+    // core may send it straight to LDS
+    static constexpr bool DIRECT = VEC;
+
     struct Ctx { unsigned off; int k; int r; };
     struct Tile { BufferRsrc rsrc; const T* p; int krem; };
 
@@ -204,12 +208,17 @@ struct DenseLoader {
         return t;
     }
 
+    // rows past the matrix edge and contraction indices past kdim read as zero
+    __device__ __forceinline__ unsigned offset(const Tile& t, const Ctx& c) const
+    {
+        return (c.k < t.krem) ? c.off : NG_OOB_OFFSET;
+    }
+
     __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const
     {
         constexpr int EPC = Elem<T>::EPC;
         if (VEC) {
-            // rows past the matrix edge and contraction indices past kdim read as zero
-            return buffer_load_chunk(t.rsrc, (c.k < t.krem) ? c.off : NG_OOB_OFFSET);
+            return buffer_load_chunk(t.rsrc, offset(t, c));
         } else {
             const T* p = t.p;
             T tmp[EPC];
@@ -480,6 +489,285 @@ void mfma_gemm_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
 }
 
 // ---------------------------------------------------------------------------
+// Direct-to-LDS variant (fp16).  Operand chunks go from global memory straight
+// into LDS (buffer_load ... lds: a wavefront instruction fills 1 KiB of LDS, lane
+// l writing bytes [16 l, 16 l + 16) after the wave-uniform base), so the tile
+// never passes through registers and NSTAGE >= 2 tiles can be in flight.
+//
+// The hardware fixes where a lane's chunk lands, so LDS tiles are unpadded and
+// bank conflicts are avoided by permuting WHICH chunk a lane fetches: the chunk
+// at position pc of line `line` holds logical chunk pc ^ swizzle(line).
+// ---------------------------------------------------------------------------
+template <typename T, int LAYOUT, int ROWS, int BK>
+struct SwizzledTile {
+    static constexpr int EPC    = Elem<T>::EPC;
+    static constexpr int CPR    = (LAYOUT == KC) ? BK / EPC : ROWS / EPC;   // chunks per line
+    static constexpr int PITCH  = CPR * 16;
+    static constexpr int LINES  = (LAYOUT == KC) ? ROWS : BK;
+    static constexpr int BYTES  = PITCH * LINES;
+    static constexpr int CHUNKS = ROWS * BK / EPC;
+    static constexpr int LP     = (CPR >= 16) ? 1 : 16 / CPR;               // lines per 256 bytes
+    static constexpr int GROUPS = (CPR / 4 < 4) ? CPR / 4 : 4;              // MC: 64-byte groups permuted
+    static_assert(sizeof(T) == 2, "direct LDS tiles are implemented for 16-bit elements");
+    static_assert(LAYOUT == MC || CPR <= 16, "contraction-contiguous lines longer than 256 bytes are not swizzled");
+    static_assert(LAYOUT == KC || CPR >= 8, "row-contiguous tiles need at least 64 rows");
+
+    // KC: 16 consecutive rows read the same logical chunk -> spread them over the
+    //     16 chunk slots of a 256-byte bank period.
+    // MC: a transposing read touches 64 contiguous bytes in each of 4 consecutive
+    //     lines -> send the 4 lines to 4 different 64-byte groups.
+    static __device__ __forceinline__ int swizzle(int line)
+    {
+        return (LAYOUT == KC) ? (line / LP) % CPR : ((line / LP) % GROUPS) * 4;
+    }
+    // LDS chunk position id (byte offset 16*id) -> first element it must hold
+    static __device__ __forceinline__ void chunk_pos(int id, int& r, int& k)
+    {
+        const int line = id / CPR, c = ((id % CPR) ^ swizzle(line)) * EPC;
+        if (LAYOUT == KC) { r = line; k = c; } else { k = line; r = c; }
+    }
+};
+
+// Fragment addressing in a swizzled tile.  base() is the lane-constant part for
+// the 32-row block `blk32` (block index inside the tile); load() adds the k-step.
+template <int LAYOUT, class Tile> struct SwizzledFrag;
+
+template <class Tile>
+struct SwizzledFrag<KC, Tile> {
+    static __device__ __forceinline__ int base(int blk32, int lane)
+    {
+        // the swizzle of row 32*b + r only depends on r
+        const int r = lane & 31;
+        return (blk32 * 32 + r) * Tile::PITCH + (((lane >> 5) ^ Tile::swizzle(r)) * 16);
+    }
+    static __device__ __forceinline__ Frag<_Float16> load(const char* tile, int base, int step)
+    {
+        // chunk index of step s is (2 s | lane>>5): the xor with the swizzle distributes
+        Frag<_Float16> f;
+        f.v = *reinterpret_cast<const half8_t*>(tile + (base ^ (step * 32)));
+        return f;
+    }
+};
+
+template <class Tile>
+struct SwizzledFrag<MC, Tile> {
+    static __device__ __forceinline__ int base(int blk32, int lane)
+    {
+        // lines step*16 + kg*8 + (l16>>2) (+4 for the second read) all share the
+        // swizzle of line kg*8 + (l16>>2)
+        const int l16 = lane & 15, blk = (lane >> 4) & 1, kg = lane >> 5;
+        const int line = kg * 8 + (l16 >> 2);
+        const int c = blk32 * 4 + blk * 2 + ((l16 >> 1) & 1);
+        return line * Tile::PITCH + ((c ^ Tile::swizzle(line)) * 16) + (l16 & 1) * 8;
+    }
+    static __device__ __forceinline__ Frag<_Float16> load(const char* tile, int base, int step)
+    {
+        const char* p = tile + base + step * 16 * Tile::PITCH;
+        short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NG_LDS short4_t*)(p));
+        short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NG_LDS short4_t*)(p + 4 * Tile::PITCH));
+        short8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        Frag<_Float16> f;
+        f.v = __builtin_bit_cast(half8_t, both);
+        return f;
+    }
+};
+
+// s_waitcnt immediate: at most `vm` vector-memory operations outstanding, all
+// LDS operations complete
+// 16 bytes per lane from a buffer straight into LDS: lane l of the wavefront
+// writes lds_base + 16 l (lds_base is wave-uniform and travels in M0); an
+// out-of-range offset stores zeros.
+//
+// Written as inline assembly on purpose.  The compiler's wait-count insertion
+// orders every LDS access it regards as a store (the transposing LDS reads are
+// among them) behind all outstanding LDS-bound loads, i.e. it would wait for the
+// tile just requested before reading the current one.  Hidden from it, these
+// loads are ordered by hand: an explicit s_waitcnt vmcnt(..) precedes the
+// barrier that publishes a stage.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void buffer_load_chunk_to_lds(BufferRsrc rsrc, char* lds_base, unsigned byte_offset)
+{
+    const unsigned lds_addr = (unsigned)(unsigned long)(NG_LDS char*)lds_base;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :: "s"(lds_addr), "v"(byte_offset), "s"(rsrc) : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
+template <int VM> struct WaitVmLgkm0 { static constexpr int IMM = (VM & 15) | ((VM >> 4) << 14) | (7 << 4); };
+
+template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, int NSTAGE,
+          class ALoad, class BLoad, class Epi>
+__global__ __launch_bounds__(WM * WN * 64)
+void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
+{
+    static_assert(ALoad::DIRECT && BLoad::DIRECT, "operands must be plain 16-byte buffer loads");
+    static_assert(NSTAGE >= 2, "need at least two LDS stages");
+    constexpr int NT = WM * WN * 64;
+    constexpr int KSTEP = Elem<T>::KSTEP;
+    using TA = SwizzledTile<T, LA, BM, BK>;
+    using TB = SwizzledTile<T, LB, BN, BK>;
+    using FA = SwizzledFrag<LA, TA>;
+    using FB = SwizzledFrag<LB, TB>;
+    constexpr int CPT_A = TA::CHUNKS / NT;
+    constexpr int CPT_B = TB::CHUNKS / NT;
+    static_assert(TA::CHUNKS % NT == 0 && TB::CHUNKS % NT == 0, "tile chunks must divide evenly over threads");
+    constexpr int TM = BM / WM / 32;
+    constexpr int TN = BN / WN / 32;
+    static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % (2 * KSTEP) == 0, "bad tile shape");
+
+    constexpr int STAGE = TA::BYTES + TB::BYTES;
+    constexpr int WTN = BN / WN;
+    constexpr int EPITCH = WTN * 4 + 16;
+    constexpr int EPI_BYTES = 32 * EPITCH;
+    constexpr int SMEM_BYTES = (NSTAGE * STAGE > EPI_BYTES * WM * WN) ? NSTAGE * STAGE : EPI_BYTES * WM * WN;
+    static_assert(SMEM_BYTES <= 160 * 1024, "tile stages exceed the LDS of a compute unit");
+    __shared__ __attribute__((aligned(16))) char smem[SMEM_BYTES];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % WM, wn = wave / WM;
+
+    int tm, tn;
+    tile_of_block(s, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int z = blockIdx.z;
+    const int split = blockIdx.y;
+
+    const int total_tiles = s.passes * s.k_tiles;
+    const int per = (total_tiles + s.splits - 1) / s.splits;
+    const int t_begin = split * per;
+    const int t_end = min(t_begin + per, total_tiles);
+    const int ntiles = t_end - t_begin;
+
+    // the chunk a lane fetches with its i-th load instruction of a tile
+    typename ALoad::Ctx actx[CPT_A];
+    typename BLoad::Ctx bctx[CPT_B];
+#pragma unroll
+    for (int i = 0; i < CPT_A; i++) { int r, k; TA::chunk_pos(tid + i * NT, r, k); actx[i] = aload.prepare(m0 + r, k); }
+#pragma unroll
+    for (int i = 0; i < CPT_B; i++) { int r, k; TB::chunk_pos(tid + i * NT, r, k); bctx[i] = bload.prepare(n0 + r, k); }
+
+    float16_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    int g_pass = t_begin / s.k_tiles;
+    int g_kt = t_begin - g_pass * s.k_tiles;
+    constexpr int NSTEP = BK / KSTEP;
+    constexpr int N_CHUNKS = CPT_A + CPT_B;
+    typename ALoad::Tile g_ta;
+    typename BLoad::Tile g_tb;
+    // fetch the next global tile into the LDS stage at byte offset `stage_off`
+    auto gissue = [&](int stage_off) {
+        g_ta = aload.tile(g_kt, g_kt * BK, z + g_pass);
+        g_tb = bload.tile(g_kt, g_kt * BK, z + g_pass);
+        if (++g_kt == s.k_tiles) { g_kt = 0; g_pass++; }
+#pragma unroll
+        for (int i = 0; i < CPT_A; i++)
+            buffer_load_chunk_to_lds(g_ta.rsrc, smem + stage_off + (i * NT + wave * 64) * 16, aload.offset(g_ta, actx[i]));
+#pragma unroll
+        for (int i = 0; i < CPT_B; i++)
+            buffer_load_chunk_to_lds(g_tb.rsrc, smem + stage_off + TA::BYTES + (i * NT + wave * 64) * 16,
+                                     bload.offset(g_tb, bctx[i]));
+    };
+
+    // lane-constant fragment addresses
+    int fa_base[TM], fb_base[TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++) fa_base[i] = FA::base(wm * TM + i, lane);
+#pragma unroll
+    for (int j = 0; j < TN; j++) fb_base[j] = TA::BYTES + FB::base(wn * TN + j, lane);
+
+    Frag<T> fa[2][TM], fb[2][TN];
+    auto load_frags = [&](int stage_off, int step, Frag<T> (&a)[TM], Frag<T> (&b)[TN]) {
+        const char* tile = smem + stage_off;
+#pragma unroll
+        for (int i = 0; i < TM; i++) a[i] = FA::load(tile, fa_base[i], step);
+#pragma unroll
+        for (int j = 0; j < TN; j++) b[j] = FB::load(tile, fb_base[j], step);
+    };
+    auto multiply = [&](const Frag<T> (&a)[TM], const Frag<T> (&b)[TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) mfma_step(a[i], b[j], acc[i][j]);
+    };
+
+    constexpr int RD_A = (LA == KC) ? 1 : 2;
+    constexpr int RD_B = (LB == KC) ? 1 : 2;
+    constexpr int N_READS = TM * RD_A + TN * RD_B;
+    constexpr int N_MFMA = TM * TN;
+    auto step = [&](int rd_stage, int rd_step, Frag<T> (&na)[TM], Frag<T> (&nb)[TN],
+                    const Frag<T> (&ca)[TM], const Frag<T> (&cb)[TN]) {
+        load_frags(rd_stage, rd_step, na, nb);
+        multiply(ca, cb);
+        InterleaveStep<0, N_MFMA, N_READS, 0>::emit();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // all k-steps of a tile but the last, fragments of the next step prefetched
+    auto head_steps = [&](int rd_stage) {
+#pragma unroll
+        for (int st = 0; st < NSTEP - 1; st++)
+            step(rd_stage, st + 1, fa[(st + 1) & 1], fb[(st + 1) & 1], fa[st & 1], fb[st & 1]);
+    };
+
+    // Pipeline.  Up to NSTAGE tiles are resident or in flight.  The iteration of
+    // tile t runs its first k-steps, waits until tile t+1 has landed, and takes
+    // the one barrier of the iteration: behind it no wavefront reads stage
+    // t % NSTAGE any more (the fragments of the last k-step are already in
+    // registers), so tile t+NSTAGE is requested into it right away and has the
+    // time of NSTAGE-1 whole tiles to arrive.  The last k-step of tile t then
+    // overlaps the first fragment reads of tile t+1.
+    auto next_stage = [&](int off) { return (off + STAGE == NSTAGE * STAGE) ? 0 : off + STAGE; };
+
+#pragma unroll
+    for (int p = 0; p < NSTAGE; p++)
+        if (p < ntiles) gissue(p * STAGE);
+    // tile 0 must have landed; the other prologue tiles may still be in flight
+    if (ntiles >= NSTAGE) __builtin_amdgcn_s_waitcnt(WaitVmLgkm0<(NSTAGE - 1) * N_CHUNKS>::IMM);
+    else                  __builtin_amdgcn_s_waitcnt(WaitVmLgkm0<0>::IMM);
+    __syncthreads();
+    int rd_off = 0;
+    if (ntiles > 0) load_frags(0, 0, fa[0], fb[0]);
+
+    int t = 0;
+    // steady state: every tile consumed frees a stage for tile t + NSTAGE
+    for (; t + NSTAGE < ntiles; t++) {
+        head_steps(rd_off);
+        __builtin_amdgcn_s_waitcnt(WaitVmLgkm0<(NSTAGE - 2) * N_CHUNKS>::IMM);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        gissue(rd_off);
+        __builtin_amdgcn_sched_barrier(0);
+        rd_off = next_stage(rd_off);
+        step(rd_off, 0, fa[NSTEP & 1], fb[NSTEP & 1], fa[(NSTEP - 1) & 1], fb[(NSTEP - 1) & 1]);
+    }
+    // drain: nothing left to request
+    for (; t + 1 < ntiles; t++) {
+        head_steps(rd_off);
+        __builtin_amdgcn_s_waitcnt(WaitVmLgkm0<0>::IMM);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        rd_off = next_stage(rd_off);
+        step(rd_off, 0, fa[NSTEP & 1], fb[NSTEP & 1], fa[(NSTEP - 1) & 1], fb[(NSTEP - 1) & 1]);
+    }
+    if (ntiles > 0) {
+        head_steps(rd_off);
+        multiply(fa[(NSTEP - 1) & 1], fb[(NSTEP - 1) & 1]);
+    }
+
+    char* stage = smem + wave * EPI_BYTES;
+    __syncthreads();
+    EpilogueBands<TM, TN, WTN, EPITCH, 0>::run(acc, stage, lane, m0 + wm * (BM / WM), n0 + wn * WTN, z, split, epi);
+}
+
+// ---------------------------------------------------------------------------
 // epilogues
 // ---------------------------------------------------------------------------
 
@@ -609,6 +897,22 @@ __global__ void splitk_reduce_kernel(const float* ws, int splits, int zcount, in
         const int i = (int)(r % m);
         const int z = (int)(r / m);
         epi.apply(i, j, z, acc);
+    }
+}
+
+// Launch the contraction core: the direct-to-LDS pipeline when both operands
+// are plain 16-byte buffer loads of 16-bit elements, the register-staged one
+// otherwise (fp32, element-wise edge handling, 8-bit inputs converted on load).
+template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, class ALoad, class BLoad, class Epi>
+inline void launch_mfma_core(dim3 grid, hipStream_t stream, const ALoad& al, const BLoad& bl, const Epi& epi,
+                             const CoreShape& s)
+{
+    if constexpr (sizeof(T) == 2 && ALoad::DIRECT && BLoad::DIRECT) {
+        hipLaunchKernelGGL((mfma_gemm_direct_kernel<T, BM, BN, BK, WM, WN, LA, LB, 2, ALoad, BLoad, Epi>), grid,
+                           dim3(WM * WN * 64), 0, stream, al, bl, epi, s);
+    } else {
+        hipLaunchKernelGGL((mfma_gemm_kernel<T, BM, BN, BK, WM, WN, LA, LB, ALoad, BLoad, Epi>), grid,
+                           dim3(WM * WN * 64), 0, stream, al, bl, epi, s);
     }
 }
 

@@ -731,11 +731,12 @@ def analyse(args):
     shape_stack = []
     values = {}
     onehots = []
+    onehot_pos = []
     max_shape = [1, 1]
     flat_size = None
     red_depth = 0
 
-    for arg in args:
+    for pos, arg in enumerate(args):
         if isinstance(arg, GPUTensor):
             if complex_op:
                 if len(arg.shape) == 2:
@@ -785,7 +786,7 @@ def analyse(args):
                 values[indx] = dict(ptr=int(arg.gpudata) if arg.gpudata is not None else 0,
                                     rs=int(strides[0]), cs=int(strides[1]), take=take_ptr,
                                     dtype=arg.dtype.str[1:], take_axis=take_axis, is_out=first_out,
-                                    itemsize=arg.dtype.itemsize)
+                                    itemsize=arg.dtype.itemsize, pos=pos)
             type_args.append(("tensor", indx))
             shape_stack.append(shape)
 
@@ -796,7 +797,7 @@ def analyse(args):
             else:
                 indx = const_ids[val] = arg_cnt
                 arg_cnt += 1
-                values[indx] = dict(const=val)
+                values[indx] = dict(const=val, pos=pos)
             type_args.append(("const", indx))
             shape_stack.append((1, 1))
 
@@ -830,6 +831,7 @@ def analyse(args):
                     hot_axis = arg["axis"] if axis else 1 - arg["axis"]
                     type_args.append(("onehot", op_cnt, hot_axis, len(onehots)))
                     onehots.append(arg["idx"].gpudata)
+                    onehot_pos.append(pos)
                     shape_stack.append(tuple(max_shape) if len(shape_stack) else (1, 1))
                 else:
                     type_args.append((op_name, op_cnt))
@@ -853,6 +855,7 @@ def analyse(args):
     plan.axis = axis
     plan.values = values
     plan.onehots = onehots
+    plan.onehot_pos = onehot_pos
     plan.type_args = type_args
 
     if not complex_op:
@@ -946,63 +949,143 @@ def analyse(args):
     return plan
 
 
+def _signature(args):
+    """Everything about a postfix stack that the analysis depends on, leaving out
+    what is merely passed through to the kernel (addresses, constant values)."""
+    from .nervanagpu import GPUTensor
+    sig = []
+    tensors, consts = {}, {}
+    for arg in args:
+        if type(arg) is dict:
+            sig.append((arg["op"], arg.get("axis", None)))
+        elif isinstance(arg, GPUTensor):
+            key = id(arg)
+            slot = tensors.get(key)
+            if slot is None:
+                slot = tensors[key] = len(tensors)
+                take = arg.take_array
+                base = arg.gpudata
+                sig.append((slot, arg.shape, arg.strides, arg.dtype.char, arg.is_trans,
+                            arg.rounding if slot == 0 else 0,
+                            take[1] if take else None,
+                            (int(base) & 15) if base is not None else 0))
+            else:
+                sig.append(slot)
+        elif type(arg) in (int, float) or isinstance(arg, (np.integer, np.floating)):
+            val = float(arg)
+            slot = consts.get(val)
+            if slot is None:
+                slot = consts[val] = len(consts)
+            sig.append(("c", slot))
+        else:
+            raise TypeError("args must be instance of GPUTensor, int, float, or dict (for operators)")
+    return tuple(sig)
+
+
+class _BoundLaunch(object):
+    """A compiled kernel with a persistent argument block.  Structurally identical
+    expressions reuse it; a call only patches the values that may differ between
+    them: addresses, constants and the random stream."""
+
+    _PTR, _TAKE, _CONST, _ONEHOT = range(4)
+
+    def __init__(self, plan, func, arg_order):
+        self.func = func
+        self.grid = (c_uint * 3)(plan.grid, 1, 1)
+        self.block = (c_uint * 3)(plan.threads, 1, 1)
+        self.empty = plan.rows == 0 or plan.n == 0
+        self.uses_rng = bool(plan.rounding) or any(a[0] == "rand" for a in plan.type_args)
+        self.shape = (plan.rows, plan.n, plan.grid, plan.threads)
+        self.patches = []
+        self.c_seed = c_uint(0)
+        self.c_stream = c_uint(0)
+        cargs = []
+        for a in arg_order:
+            kind = a[0]
+            if kind == "ptr":
+                c = c_void_p(plan.values[a[1]]["ptr"])
+                self.patches.append((c, self._PTR, plan.values[a[1]]["pos"]))
+            elif kind == "rs":
+                c = c_int(plan.values[a[1]]["rs"])
+            elif kind == "cs":
+                c = c_int(plan.values[a[1]]["cs"])
+            elif kind == "take":
+                c = c_void_p(int(plan.values[a[1]]["take"]))
+                self.patches.append((c, self._TAKE, plan.values[a[1]]["pos"]))
+            elif kind == "const":
+                c = c_float(plan.values[a[1]]["const"])
+                self.patches.append((c, self._CONST, plan.values[a[1]]["pos"]))
+            elif kind == "onehot":
+                c = c_void_p(int(plan.onehots[a[1]]))
+                self.patches.append((c, self._ONEHOT, plan.onehot_pos[a[1]]))
+            elif kind == "n":
+                c = c_int(plan.n)
+            elif kind == "n_out":
+                c = c_int(plan.n_out)
+            elif kind == "rows":
+                c = ctypes.c_long(plan.rows)
+            elif kind == "sr_bits":
+                c = c_uint(plan.rounding)
+            elif kind == "rng_seed":
+                c = self.c_seed
+            elif kind == "rng_stream":
+                c = self.c_stream
+            elif kind == "rng_rm":
+                c = c_uint(plan.rng_rm)
+            elif kind == "rng_cm":
+                c = c_uint(plan.rng_cm)
+            else:
+                raise AssertionError(kind)
+            cargs.append(c)
+        self.cargs = cargs          # keeps the storage the pointer block refers to alive
+        self.ptrs = (c_void_p * len(cargs))(*[ctypes.addressof(c) for c in cargs])
+        self.entry = _lib.load().ng_launch
+
+    def __call__(self, backend, args):
+        if self.empty:
+            return
+        for c, kind, pos in self.patches:
+            a = args[pos]
+            if kind == 0:
+                base = a.gpudata
+                c.value = int(base) if base is not None else 0
+            elif kind == 2:
+                c.value = float(a)
+            elif kind == 1:
+                c.value = int(a.take_array[0].gpudata)
+            else:
+                c.value = int(a["idx"].gpudata)
+        if self.uses_rng:
+            self.c_seed.value, self.c_stream.value = backend._next_rng_stream()
+        repeat = backend.bench if isinstance(backend.bench, int) and backend.bench > 1 else 1
+        if repeat > 1:
+            start, end = backend._get_events()
+            start.record(backend.stream)
+        for _ in range(repeat):
+            _lib.check(self.entry(self.func.handle, self.grid, self.block, 0, backend.stream, self.ptrs))
+        if repeat > 1:
+            end.record(backend.stream)
+            end.synchronize()
+            msecs = end.time_since(start) / repeat
+            backend.last_bench_msecs = msecs
+            print("%7.3f msecs shape(%d,%d) blk,thd(%d,%d) %s" % ((msecs,) + self.shape + (self.func.name,)))
+
+
+_bound_cache = {}
+
+
 def call_compound_kernel(backend, *args):
     """Execute a postfix expression stack ending in {"op": "assign"}:
         C += 2.5 * A * B + 1  ==  (C, 2.5, A, mul, B, mul, 1, add, C, add, assign)
     `backend` supplies the stream and the random stream (seed, launch counter).
     Returns the output tensor (nervanagpu/float_ew.py:1058-1322)."""
-    plan = analyse(args)
-    out = plan.out
-    if plan.rows == 0 or plan.n == 0:
-        return out
-    func, arg_order, _ = _get_kernel(plan.spec)
-
-    rounding = plan.rounding
-    uses_rng = rounding or any(a[0] == "rand" for a in plan.type_args)
-    seed, stream_id = backend._next_rng_stream() if uses_rng else (0, 0)
-
-    cargs = []
-    for a in arg_order:
-        kind = a[0]
-        if kind == "ptr":
-            cargs.append(c_void_p(plan.values[a[1]]["ptr"]))
-        elif kind == "rs":
-            cargs.append(c_int(plan.values[a[1]]["rs"]))
-        elif kind == "cs":
-            cargs.append(c_int(plan.values[a[1]]["cs"]))
-        elif kind == "take":
-            cargs.append(c_void_p(int(plan.values[a[1]]["take"])))
-        elif kind == "const":
-            cargs.append(c_float(plan.values[a[1]]["const"]))
-        elif kind == "onehot":
-            cargs.append(c_void_p(int(plan.onehots[a[1]])))
-        elif kind == "n":
-            cargs.append(c_int(plan.n))
-        elif kind == "n_out":
-            cargs.append(c_int(plan.n_out))
-        elif kind == "rows":
-            cargs.append(ctypes.c_long(plan.rows))
-        elif kind == "sr_bits":
-            cargs.append(c_uint(rounding))
-        elif kind == "rng_seed":
-            cargs.append(c_uint(seed))
-        elif kind == "rng_stream":
-            cargs.append(c_uint(stream_id))
-        elif kind == "rng_rm":
-            cargs.append(c_uint(plan.rng_rm))
-        elif kind == "rng_cm":
-            cargs.append(c_uint(plan.rng_cm))
-
-    repeat = backend.bench if isinstance(backend.bench, int) and backend.bench > 1 else 1
-    if repeat > 1:
-        start, end = backend._get_events()
-        start.record(backend.stream)
-    for _ in range(repeat):
-        func.launch((plan.grid, 1, 1), (plan.threads, 1, 1), backend.stream, cargs)
-    if repeat > 1:
-        end.record(backend.stream)
-        end.synchronize()
-        msecs = end.time_since(start) / repeat
-        print("%7.3f msecs shape(%d,%d) blk,thd(%d,%d) %s" %
-              (msecs, plan.rows, plan.n, plan.grid, plan.threads, func.name))
-    return out
+    sig = _signature(args)
+    bound = _bound_cache.get(sig)
+    if bound is None:
+        plan = analyse(args)
+        if plan.rows == 0 or plan.n == 0:
+            return plan.out
+        func, arg_order, _ = _get_kernel(plan.spec)
+        bound = _bound_cache[sig] = _BoundLaunch(plan, func, arg_order)
+    bound(backend, args)
+    return args[0]
