@@ -36,26 +36,6 @@ struct TapEntry { int off, dz, dy, dx; };
 typedef unsigned char u8_t;
 typedef signed char   s8_t;
 
-// n / d for 0 <= n < 2^31 as a multiply and a shift.  With s = ceil(log2 d),
-// mul = floor(2^(31+s) / d) + 1 fits 32 bits and the quotient is exact because
-// the rounding excess n * (mul*d - 2^(31+s)) stays below 2^(31+s).
-struct FastDiv {
-    unsigned mul, shift;
-    __host__ __device__ __forceinline__ unsigned div(unsigned n) const
-    {
-        return (unsigned)(((unsigned long long)n * mul) >> shift);
-    }
-    static FastDiv make(unsigned d)
-    {
-        unsigned s = 0;
-        while ((1ull << s) < d) s++;
-        FastDiv f;
-        f.mul = (unsigned)((1ull << (31 + s)) / d + 1);
-        f.shift = 31 + s;
-        return f;
-    }
-};
-
 // 16-byte chunk of compute type T from storage type TIN via a raw buffer load
 template <typename T, typename TIN> struct ChunkFetch;
 

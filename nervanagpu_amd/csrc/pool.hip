@@ -55,26 +55,48 @@ struct PoolGeom {
     int pad_j, pad_d, pad_h, pad_w;
     int str_j, str_d, str_h, str_w;
     int nvec;           // N / VEC
+    // index decomposition without integer division: a thread's position inside
+    // one feature map is split by nvec, then by the two inner spatial extents
+    // (fprop kernels: Q, P; bprop gather: W, H); window ranges divide by strides
+    FastDiv div_nvec, div_q, div_p, div_w, div_h;
+    FastDiv div_sj, div_sd, div_sh, div_sw;
 };
 
 enum { OP_MAX = 0, OP_AVG = 1 };
 
 #define NG_FLT_MAX 3.402823466e+38f
 
-// one thread: VEC images of one output element
-template <typename T, int VEC, int OP, bool WRITE_ARG>
+// Launch geometry shared by the kernels: blockIdx.y is the outermost index
+// (output or input feature map), blockIdx.x * 256 + threadIdx.x the position
+// inside that map: ((d * H + h) * W + w) * nvec + nv, below 2^31.
+__device__ __forceinline__ bool split_inner(unsigned inner, unsigned limit, const FastDiv& dn, const FastDiv& d1,
+                                            const FastDiv& d2, int nvec, int e1, int e2, int& nv, int& i1, int& i2,
+                                            int& i3)
+{
+    if (inner >= limit) return false;
+    unsigned r = dn.div(inner);
+    nv = (int)(inner - r * (unsigned)nvec);
+    unsigned r1 = d1.div(r);
+    i1 = (int)(r - r1 * (unsigned)e1);
+    unsigned r2 = d2.div(r1);
+    i2 = (int)(r1 - r2 * (unsigned)e2);
+    i3 = (int)r2;
+    return true;
+}
+
+// one thread: VEC images of one output element.  RS > 0: the window is a 2-D
+// RS x RS square (J == T == 1), known at compile time, so all its loads are
+// issued together; taps outside the image are redirected to a valid address and
+// replaced by the identity of the reduction.
+template <typename T, int VEC, int OP, bool WRITE_ARG, int RS>
 __global__ __launch_bounds__(256)
 void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char* __restrict__ arg, PoolGeom g)
 {
-    const long total = (long)g.K * g.M * g.P * g.Q * g.nvec;
-    const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= total) return;
-    const int nv = (int)(e % g.nvec);
-    long r = e / g.nvec;
-    const int q = (int)(r % g.Q); r /= g.Q;
-    const int p = (int)(r % g.P); r /= g.P;
-    const int m = (int)(r % g.M);
-    const int k = (int)(r / g.M);
+    const unsigned per_map = (unsigned)(g.M * g.P * g.Q * g.nvec);
+    const unsigned inner = blockIdx.x * 256u + threadIdx.x;
+    const int k = blockIdx.y;
+    int nv, q, p, m;
+    if (!split_inner(inner, per_map, g.div_nvec, g.div_q, g.div_p, g.nvec, g.Q, g.P, nv, q, p, m)) return;
     const int c0 = k * g.str_j - g.pad_j, z0 = m * g.str_d - g.pad_d;
     const int y0 = p * g.str_h - g.pad_h, x0 = q * g.str_w - g.pad_w;
 
@@ -83,25 +105,58 @@ void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char
 #pragma unroll
     for (int i = 0; i < VEC; i++) { best[i] = (OP == OP_MAX) ? -NG_FLT_MAX : 0.0f; slot_of[i] = 0; }
 
-    int slot = 0;
-    for (int j = 0; j < g.J; j++) {
-        const int c = c0 + j;
-        for (int t = 0; t < g.T; t++) {
-            const int z = z0 + t;
-            for (int rr = 0; rr < g.R; rr++) {
-                const int y = y0 + rr;
-                for (int s = 0; s < g.S; s++, slot++) {
-                    const int x = x0 + s;
-                    if ((unsigned)c < (unsigned)g.C && (unsigned)z < (unsigned)g.D &&
-                        (unsigned)y < (unsigned)g.H && (unsigned)x < (unsigned)g.W) {
-                        float v[VEC];
-                        load_vec<T, VEC>(I + ((((long)c * g.D + z) * g.H + y) * g.W + x) * g.N + (long)nv * VEC, v);
+    const T* Inv = I + (long)nv * VEC;
+    if (RS > 0) {
+        constexpr int NTAP = RS > 0 ? RS * RS : 1;
+        const bool plane_ok = (unsigned)c0 < (unsigned)g.C && (unsigned)z0 < (unsigned)g.D;
+        const T* plane = Inv + ((long)c0 * g.D + z0) * g.H * g.W * g.N;
+        typedef typename Pack<T, VEC>::raw_t raw_t;
+        raw_t raw[NTAP];
+        bool ok[NTAP];
 #pragma unroll
-                        for (int i = 0; i < VEC; i++) {
-                            if (OP == OP_MAX) {
-                                if (v[i] > best[i]) { best[i] = v[i]; slot_of[i] = slot; }
-                            } else {
-                                best[i] += v[i];
+        for (int tap = 0; tap < NTAP; tap++) {
+            const int y = y0 + tap / (RS > 0 ? RS : 1), x = x0 + tap % (RS > 0 ? RS : 1);
+            ok[tap] = plane_ok && (unsigned)y < (unsigned)g.H && (unsigned)x < (unsigned)g.W;
+            const T* src = ok[tap] ? plane + ((long)y * g.W + x) * g.N : Inv;
+            raw[tap] = *reinterpret_cast<const raw_t*>(src);
+        }
+#pragma unroll
+        for (int tap = 0; tap < NTAP; tap++) {
+            const T* e = reinterpret_cast<const T*>(&raw[tap]);
+#pragma unroll
+            for (int i = 0; i < VEC; i++) {
+                const float v = (float)e[i];
+                if (OP == OP_MAX) {
+                    if (ok[tap] && v > best[i]) { best[i] = v; slot_of[i] = tap; }
+                } else {
+                    best[i] += ok[tap] ? v : 0.0f;
+                }
+            }
+        }
+    } else {
+        int slot = 0;
+        for (int j = 0; j < g.J; j++) {
+            const int c = c0 + j;
+            for (int t = 0; t < g.T; t++) {
+                const int z = z0 + t;
+                const bool plane_ok = (unsigned)c < (unsigned)g.C && (unsigned)z < (unsigned)g.D;
+                const long plane = ((long)c * g.D + z) * g.H;
+                for (int rr = 0; rr < g.R; rr++) {
+                    const int y = y0 + rr;
+                    const bool row_ok = plane_ok && (unsigned)y < (unsigned)g.H;
+                    const T* row = Inv + (plane + y) * g.W * g.N;
+                    for (int s = 0; s < g.S; s++, slot++) {
+                        const int x = x0 + s;
+                        if (row_ok && (unsigned)x < (unsigned)g.W) {
+                            float v[VEC];
+                            load_vec<T, VEC>(row + (long)x * g.N, v);
+#pragma unroll
+                            for (int i = 0; i < VEC; i++) {
+                                if (OP == OP_MAX) {
+                                    if (v[i] > best[i]) { best[i] = v[i]; slot_of[i] = slot; }
+                                } else {
+                                    best[i] += v[i];
+                                }
                             }
                         }
                     }
@@ -109,10 +164,18 @@ void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char
             }
         }
     }
-    const long o = e * VEC;
+    const long o = ((long)k * per_map + inner) * VEC;
     if (WRITE_ARG) {
+        if (VEC == 8) {
+            uint2 packed;
+            packed.x = (unsigned)slot_of[0] | ((unsigned)slot_of[1] << 8) | ((unsigned)slot_of[2] << 16) | ((unsigned)slot_of[3] << 24);
+            packed.y = (unsigned)slot_of[4 % VEC] | ((unsigned)slot_of[5 % VEC] << 8) | ((unsigned)slot_of[6 % VEC] << 16) |
+                       ((unsigned)slot_of[7 % VEC] << 24);
+            *reinterpret_cast<uint2*>(arg + o) = packed;
+        } else {
 #pragma unroll
-        for (int i = 0; i < VEC; i++) arg[o + i] = (unsigned char)slot_of[i];
+            for (int i = 0; i < VEC; i++) arg[o + i] = (unsigned char)slot_of[i];
+        }
     } else {
         if (OP == OP_AVG) {
             const float inv = 1.0f / (float)(g.J * g.T * g.R * g.S);
@@ -123,74 +186,118 @@ void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char
     }
 }
 
-__device__ __forceinline__ void window_range(int coord, int pad, int win, int str, int count, int& lo, int& hi)
+__device__ __forceinline__ void window_range(int coord, int pad, int win, int str, const FastDiv& dstr, int count,
+                                             int& lo, int& hi)
 {
     // outputs o with o*str - pad <= coord <= o*str - pad + win - 1
     const int a = coord + pad - win + 1;
-    lo = a <= 0 ? 0 : (a + str - 1) / str;
-    hi = (coord + pad) / str;
+    lo = a <= 0 ? 0 : (int)dstr.div((unsigned)(a + str - 1));
+    hi = (int)dstr.div((unsigned)(coord + pad));
     if (hi > count - 1) hi = count - 1;
 }
 
-// one thread: VEC images of one input element; sums the errors of the covering
-// windows in a fixed (k,m,p,q) order
+// accumulate the error of one covering window into acc
 template <typename T, int VEC, int OP>
+__device__ __forceinline__ void add_window(float (&acc)[VEC], const typename Pack<T, VEC>::raw_t& eraw, uint2 a, int slot,
+                                           bool valid)
+{
+    const T* ev = reinterpret_cast<const T*>(&eraw);
+    if (OP == OP_MAX) {
+#pragma unroll
+        for (int i = 0; i < VEC; i++) {
+            const unsigned word = (i < 4) ? a.x : a.y;
+            const int s = (int)((word >> (8 * (i & 3))) & 0xFF);
+            acc[i] += (valid && s == slot) ? (float)ev[i] : 0.0f;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < VEC; i++) acc[i] += valid ? (float)ev[i] : 0.0f;
+    }
+}
+
+// one thread: VEC images of one input element; sums the errors of the covering
+// windows in a fixed (k,m,p,q) order.  WIN2: at most two windows cover an
+// element along h and along w, and one along c and d; the (up to) four loads
+// are then issued together instead of inside data-dependent loops.
+template <typename T, int VEC, int OP, bool WIN2>
 __global__ __launch_bounds__(256)
 void pool_bprop_kernel(const T* __restrict__ E, const unsigned char* __restrict__ arg, T* __restrict__ B, PoolGeom g)
 {
-    const long total = (long)g.C * g.D * g.H * g.W * g.nvec;
-    const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= total) return;
-    const int nv = (int)(e % g.nvec);
-    long r = e / g.nvec;
-    const int x = (int)(r % g.W); r /= g.W;
-    const int y = (int)(r % g.H); r /= g.H;
-    const int z = (int)(r % g.D);
-    const int c = (int)(r / g.D);
+    const unsigned per_map = (unsigned)(g.D * g.H * g.W * g.nvec);
+    const unsigned inner = blockIdx.x * 256u + threadIdx.x;
+    const int c = blockIdx.y;
+    int nv, x, y, z;
+    if (!split_inner(inner, per_map, g.div_nvec, g.div_w, g.div_h, g.nvec, g.W, g.H, nv, x, y, z)) return;
 
     int k0, k1, m0, m1, p0, p1, q0, q1;
-    window_range(c, g.pad_j, g.J, g.str_j, g.K, k0, k1);
-    window_range(z, g.pad_d, g.T, g.str_d, g.M, m0, m1);
-    window_range(y, g.pad_h, g.R, g.str_h, g.P, p0, p1);
-    window_range(x, g.pad_w, g.S, g.str_w, g.Q, q0, q1);
+    window_range(c, g.pad_j, g.J, g.str_j, g.div_sj, g.K, k0, k1);
+    window_range(z, g.pad_d, g.T, g.str_d, g.div_sd, g.M, m0, m1);
+    window_range(y, g.pad_h, g.R, g.str_h, g.div_sh, g.P, p0, p1);
+    window_range(x, g.pad_w, g.S, g.str_w, g.div_sw, g.Q, q0, q1);
 
     float acc[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; i++) acc[i] = 0.0f;
 
-    for (int k = k0; k <= k1; k++)
-        for (int m = m0; m <= m1; m++)
-            for (int p = p0; p <= p1; p++)
-                for (int q = q0; q <= q1; q++) {
-                    const long o = (((((long)k * g.M + m) * g.P + p) * g.Q + q) * g.nvec + nv) * VEC;
-                    float ev[VEC];
-                    load_vec<T, VEC>(E + o, ev);
-                    if (OP == OP_MAX) {
-                        const int slot = (((c - (k * g.str_j - g.pad_j)) * g.T + (z - (m * g.str_d - g.pad_d))) * g.R +
-                                          (y - (p * g.str_h - g.pad_h))) * g.S + (x - (q * g.str_w - g.pad_w));
-                        if (VEC == 8) {
-                            const uint2 a = *reinterpret_cast<const uint2*>(arg + o);
+    if (WIN2 && VEC == 8) {
+        typedef typename Pack<T, VEC>::raw_t raw_t;
+        const bool km_ok = k0 <= k1 && m0 <= m1;
+        const int k = k0, m = m0;
+        const int slot_km = ((c - (k * g.str_j - g.pad_j)) * g.T + (z - (m * g.str_d - g.pad_d))) * g.R;
+        raw_t eraw[4];
+        uint2 a[4];
+        bool ok[4];
+        int slot[4];
 #pragma unroll
-                            for (int i = 0; i < 4; i++) {
-                                if ((int)((a.x >> (8 * i)) & 0xFF) == slot) acc[i] += ev[i];
-                                if ((int)((a.y >> (8 * i)) & 0xFF) == slot) acc[(i + 4) % VEC] += ev[(i + 4) % VEC];
+        for (int w = 0; w < 4; w++) {
+            const int p = p0 + (w >> 1), q = q0 + (w & 1);
+            ok[w] = km_ok && p <= p1 && q <= q1;
+            const long o = ok[w] ? (((((long)k * g.M + m) * g.P + p) * g.Q + q) * g.nvec + nv) * VEC : (long)nv * VEC;
+            eraw[w] = *reinterpret_cast<const raw_t*>(E + o);
+            a[w] = (OP == OP_MAX) ? *reinterpret_cast<const uint2*>(arg + o) : make_uint2(0, 0);
+            slot[w] = (slot_km + (y - (p * g.str_h - g.pad_h))) * g.S + (x - (q * g.str_w - g.pad_w));
+        }
+#pragma unroll
+        for (int w = 0; w < 4; w++) add_window<T, VEC, OP>(acc, eraw[w], a[w], slot[w], ok[w]);
+    } else {
+        for (int k = k0; k <= k1; k++)
+            for (int m = m0; m <= m1; m++) {
+                const int slot_km = ((c - (k * g.str_j - g.pad_j)) * g.T + (z - (m * g.str_d - g.pad_d))) * g.R;
+                for (int p = p0; p <= p1; p++) {
+                    const int slot_p = (slot_km + (y - (p * g.str_h - g.pad_h))) * g.S + x + g.pad_w;
+                    const long row = ((((long)k * g.M + m) * g.P + p) * g.Q * g.nvec + nv) * VEC;
+                    for (int q = q0; q <= q1; q++) {
+                        const long o = row + (long)q * g.nvec * VEC;
+                        float ev[VEC];
+                        load_vec<T, VEC>(E + o, ev);
+                        if (OP == OP_MAX) {
+                            const int slot = slot_p - q * g.str_w;
+                            if (VEC == 8) {
+                                const uint2 a = *reinterpret_cast<const uint2*>(arg + o);
+#pragma unroll
+                                for (int i = 0; i < 4; i++) {
+                                    if ((int)((a.x >> (8 * i)) & 0xFF) == slot) acc[i] += ev[i];
+                                    if ((int)((a.y >> (8 * i)) & 0xFF) == slot) acc[(i + 4) % VEC] += ev[(i + 4) % VEC];
+                                }
+                            } else {
+#pragma unroll
+                                for (int i = 0; i < VEC; i++)
+                                    if ((int)arg[o + i] == slot) acc[i] += ev[i];
                             }
                         } else {
 #pragma unroll
-                            for (int i = 0; i < VEC; i++)
-                                if ((int)arg[o + i] == slot) acc[i] += ev[i];
+                            for (int i = 0; i < VEC; i++) acc[i] += ev[i];
                         }
-                    } else {
-#pragma unroll
-                        for (int i = 0; i < VEC; i++) acc[i] += ev[i];
                     }
                 }
+            }
+    }
     if (OP == OP_AVG) {
         const float inv = 1.0f / (float)(g.J * g.T * g.R * g.S);
 #pragma unroll
         for (int i = 0; i < VEC; i++) acc[i] *= inv;
     }
-    store_vec<T, VEC>(B + e * VEC, acc);
+    store_vec<T, VEC>(B + ((long)c * per_map + inner) * VEC, acc);
 }
 
 // windows that tile the input exactly (stride == window, no padding, extents
@@ -200,16 +307,14 @@ template <typename T, int VEC>
 __global__ __launch_bounds__(256)
 void pool_bprop_max_tiled_kernel(const T* __restrict__ I, const T* __restrict__ E, T* __restrict__ B, PoolGeom g)
 {
-    const long total = (long)g.K * g.M * g.P * g.Q * g.nvec;
-    const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= total) return;
-    const int nv = (int)(e % g.nvec);
-    long r = e / g.nvec;
-    const int q = (int)(r % g.Q); r /= g.Q;
-    const int p = (int)(r % g.P); r /= g.P;
-    const int m = (int)(r % g.M);
-    const int k = (int)(r / g.M);
+    const unsigned per_map = (unsigned)(g.M * g.P * g.Q * g.nvec);
+    const unsigned inner = blockIdx.x * 256u + threadIdx.x;
+    const int k = blockIdx.y;
+    int nv, q, p, m;
+    if (!split_inner(inner, per_map, g.div_nvec, g.div_q, g.div_p, g.nvec, g.Q, g.P, nv, q, p, m)) return;
     const int c0 = k * g.J, z0 = m * g.T, y0 = p * g.R, x0 = q * g.S;
+    const long in_base = ((((long)c0 * g.D + z0) * g.H + y0) * g.W + x0) * g.N + (long)nv * VEC;
+    const long sx = g.N, sy = (long)g.W * g.N, sz = (long)g.H * g.W * g.N, sc = (long)g.D * g.H * g.W * g.N;
 
     float best[VEC];
     int   slot_of[VEC];
@@ -221,14 +326,13 @@ void pool_bprop_max_tiled_kernel(const T* __restrict__ I, const T* __restrict__ 
             for (int rr = 0; rr < g.R; rr++)
                 for (int s = 0; s < g.S; s++, slot++) {
                     float v[VEC];
-                    load_vec<T, VEC>(I + ((((long)(c0 + j) * g.D + z0 + t) * g.H + y0 + rr) * g.W + x0 + s) * g.N +
-                                         (long)nv * VEC, v);
+                    load_vec<T, VEC>(I + in_base + j * sc + t * sz + rr * sy + s * sx, v);
 #pragma unroll
                     for (int i = 0; i < VEC; i++)
                         if (v[i] > best[i]) { best[i] = v[i]; slot_of[i] = slot; }
                 }
     float ev[VEC];
-    load_vec<T, VEC>(E + e * VEC, ev);
+    load_vec<T, VEC>(E + ((long)k * per_map + inner) * VEC, ev);
     slot = 0;
     for (int j = 0; j < g.J; j++)
         for (int t = 0; t < g.T; t++)
@@ -237,8 +341,7 @@ void pool_bprop_max_tiled_kernel(const T* __restrict__ I, const T* __restrict__ 
                     float out[VEC];
 #pragma unroll
                     for (int i = 0; i < VEC; i++) out[i] = (slot_of[i] == slot) ? ev[i] : 0.0f;
-                    store_vec<T, VEC>(B + ((((long)(c0 + j) * g.D + z0 + t) * g.H + y0 + rr) * g.W + x0 + s) * g.N +
-                                          (long)nv * VEC, out);
+                    store_vec<T, VEC>(B + in_base + j * sc + t * sz + rr * sy + s * sx, out);
                 }
 }
 
@@ -246,6 +349,15 @@ static PoolGeom make_geom(const ng_pool_params& p, int vec)
 {
     PoolGeom g{p.N, p.C, p.D, p.H, p.W, p.J, p.T, p.R, p.S, p.K, p.M, p.P, p.Q,
                p.pad_j, p.pad_d, p.pad_h, p.pad_w, p.str_j, p.str_d, p.str_h, p.str_w, p.N / vec};
+    g.div_nvec = FastDiv::make((unsigned)g.nvec);
+    g.div_q = FastDiv::make((unsigned)p.Q);
+    g.div_p = FastDiv::make((unsigned)p.P);
+    g.div_w = FastDiv::make((unsigned)p.W);
+    g.div_h = FastDiv::make((unsigned)p.H);
+    g.div_sj = FastDiv::make((unsigned)p.str_j);
+    g.div_sd = FastDiv::make((unsigned)p.str_d);
+    g.div_sh = FastDiv::make((unsigned)p.str_h);
+    g.div_sw = FastDiv::make((unsigned)p.str_w);
     return g;
 }
 
@@ -262,24 +374,61 @@ static int check_params(const ng_pool_params& p, int dtype, int op)
     if (op != OP_MAX && op != OP_AVG) return fail(-61, "pool: op must be 0 (max) or 1 (avg)");
     if (p.N <= 0 || p.C <= 0 || p.K <= 0 || p.M <= 0 || p.P <= 0 || p.Q <= 0) return fail(-62, "pool: empty geometry");
     if (p.str_j < 1 || p.str_d < 1 || p.str_h < 1 || p.str_w < 1) return fail(-63, "pool: strides must be >= 1");
+    if (p.D <= 0 || p.H <= 0 || p.W <= 0) return fail(-62, "pool: empty geometry");
+    // one feature map is indexed with 31 bits, feature maps with gridDim.y
+    if ((long)p.D * p.H * p.W * p.N >= (1L << 31) || (long)p.M * p.P * p.Q * p.N >= (1L << 31))
+        return fail(-67, "pool: a single feature map must hold fewer than 2^31 elements");
+    if (p.C > 65535 || p.K > 65535) return fail(-68, "pool: more than 65535 feature maps are not supported");
     return 0;
 }
 
-static unsigned blocks_for(long total) { return (unsigned)((total + 255) / 256); }
+// grid over (positions of one feature map) x (feature maps)
+static dim3 grid_for(long per_map, int maps) { return dim3((unsigned)((per_map + 255) / 256), (unsigned)maps, 1); }
+
+// compile-time window size of the unrolled forward kernels (0: generic loops)
+static int square_window(const ng_pool_params& p)
+{
+    if (p.J != 1 || p.T != 1 || p.R != p.S) return 0;
+    return (p.R == 2 || p.R == 3) ? p.R : 0;
+}
+
+template <typename T, int VEC, int OP, bool WRITE_ARG>
+static void launch_fprop(const PoolGeom& g, int rs, dim3 grid, const T* I, T* O, unsigned char* arg, hipStream_t st)
+{
+    if (rs == 2 && VEC > 1)
+        hipLaunchKernelGGL((pool_fprop_kernel<T, VEC, OP, WRITE_ARG, 2>), grid, dim3(256), 0, st, I, O, arg, g);
+    else if (rs == 3 && VEC > 1)
+        hipLaunchKernelGGL((pool_fprop_kernel<T, VEC, OP, WRITE_ARG, 3>), grid, dim3(256), 0, st, I, O, arg, g);
+    else
+        hipLaunchKernelGGL((pool_fprop_kernel<T, VEC, OP, WRITE_ARG, 0>), grid, dim3(256), 0, st, I, O, arg, g);
+}
 
 template <typename T, int VEC>
 static int run_fprop(const ng_pool_params& p, int op, const void* I, void* O, hipStream_t st)
 {
     PoolGeom g = make_geom(p, VEC);
-    const long total = (long)g.K * g.M * g.P * g.Q * g.nvec;
-    if (op == OP_MAX)
-        hipLaunchKernelGGL((pool_fprop_kernel<T, VEC, OP_MAX, false>), dim3(blocks_for(total)), dim3(256), 0, st,
-                           (const T*)I, (T*)O, (unsigned char*)nullptr, g);
-    else
-        hipLaunchKernelGGL((pool_fprop_kernel<T, VEC, OP_AVG, false>), dim3(blocks_for(total)), dim3(256), 0, st,
-                           (const T*)I, (T*)O, (unsigned char*)nullptr, g);
+    const dim3 grid = grid_for((long)g.M * g.P * g.Q * g.nvec, g.K);
+    const int rs = square_window(p);
+    if (op == OP_MAX) launch_fprop<T, VEC, OP_MAX, false>(g, rs, grid, (const T*)I, (T*)O, nullptr, st);
+    else              launch_fprop<T, VEC, OP_AVG, false>(g, rs, grid, (const T*)I, (T*)O, nullptr, st);
     NG_CHECK_LAUNCH("pool fprop");
     return 0;
+}
+
+// at most two covering windows along h and w and one along c and d
+static bool two_window_cover(const ng_pool_params& p)
+{
+    return p.J == 1 && p.T == 1 && (p.R + p.str_h - 1) / p.str_h <= 2 && (p.S + p.str_w - 1) / p.str_w <= 2;
+}
+
+template <typename T, int VEC, int OP>
+static void launch_gather(const PoolGeom& g, bool win2, dim3 grid, const T* E, const unsigned char* arg, T* B,
+                          hipStream_t st)
+{
+    if (win2 && VEC == 8)
+        hipLaunchKernelGGL((pool_bprop_kernel<T, VEC, OP, true>), grid, dim3(256), 0, st, E, arg, B, g);
+    else
+        hipLaunchKernelGGL((pool_bprop_kernel<T, VEC, OP, false>), grid, dim3(256), 0, st, E, arg, B, g);
 }
 
 template <typename T, int VEC>
@@ -288,15 +437,16 @@ static int run_bprop(const ng_pool_params& p, int op, const void* I, const void*
 {
     PoolGeom g = make_geom(p, VEC);
     const long out_total = (long)g.K * g.M * g.P * g.Q * g.nvec;
-    const long in_total = (long)g.C * g.D * g.H * g.W * g.nvec;
+    const dim3 out_grid = grid_for((long)g.M * g.P * g.Q * g.nvec, g.K);
+    const dim3 in_grid = grid_for((long)g.D * g.H * g.W * g.nvec, g.C);
+    const bool win2 = two_window_cover(p);
     if (op == OP_AVG) {
-        hipLaunchKernelGGL((pool_bprop_kernel<T, VEC, OP_AVG>), dim3(blocks_for(in_total)), dim3(256), 0, st,
-                           (const T*)E, (const unsigned char*)nullptr, (T*)B, g);
+        launch_gather<T, VEC, OP_AVG>(g, win2, in_grid, (const T*)E, nullptr, (T*)B, st);
         NG_CHECK_LAUNCH("pool avg bprop");
         return 0;
     }
     if (tiles_exactly(p)) {
-        hipLaunchKernelGGL((pool_bprop_max_tiled_kernel<T, VEC>), dim3(blocks_for(out_total)), dim3(256), 0, st,
+        hipLaunchKernelGGL((pool_bprop_max_tiled_kernel<T, VEC>), out_grid, dim3(256), 0, st,
                            (const T*)I, (const T*)E, (T*)B, g);
         NG_CHECK_LAUNCH("pool max bprop (tiled)");
         return 0;
@@ -304,11 +454,9 @@ static int run_bprop(const ng_pool_params& p, int op, const void* I, const void*
     const size_t need = (size_t)out_total * VEC;
     if (!ws || ws_bytes < need) return fail(-64, "pool max bprop: workspace too small (%zu < %zu)", ws_bytes, need);
     if (p.J * p.T * p.R * p.S > 256) return fail(-65, "pool max bprop: windows of more than 256 elements are not supported");
-    hipLaunchKernelGGL((pool_fprop_kernel<T, VEC, OP_MAX, true>), dim3(blocks_for(out_total)), dim3(256), 0, st,
-                       (const T*)I, (T*)nullptr, (unsigned char*)ws, g);
+    launch_fprop<T, VEC, OP_MAX, true>(g, square_window(p), out_grid, (const T*)I, (T*)nullptr, (unsigned char*)ws, st);
     NG_CHECK_LAUNCH("pool argmax");
-    hipLaunchKernelGGL((pool_bprop_kernel<T, VEC, OP_MAX>), dim3(blocks_for(in_total)), dim3(256), 0, st,
-                       (const T*)E, (const unsigned char*)ws, (T*)B, g);
+    launch_gather<T, VEC, OP_MAX>(g, win2, in_grid, (const T*)E, (const unsigned char*)ws, (T*)B, st);
     NG_CHECK_LAUNCH("pool max bprop");
     return 0;
 }

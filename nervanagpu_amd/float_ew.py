@@ -33,13 +33,16 @@ import numpy as np
 
 from . import _lib
 
-# op name -> (operand count, C expression); {0},{1} are the operands in source order
+# op name -> (operand count, C expression); {0},{1} are the operands in source order.
+# The reference builds its kernels with --use_fast_math (nervanagpu/float_ew.py:1030):
+# division and square root are the hardware approximations (about 1 ulp), not
+# the correctly rounded sequences.
 _float_ops = {
     "assign":  (2, None),
     "add":     (2, "({0} + {1})"),
     "sub":     (2, "({0} - {1})"),
     "mul":     (2, "({0} * {1})"),
-    "div":     (2, "({0} / {1})"),
+    "div":     (2, "({0} * __builtin_amdgcn_rcpf({1}))"),
     "eq":      (2, "(({0} == {1}) ? 1.0f : 0.0f)"),
     "ne":      (2, "(({0} != {1}) ? 1.0f : 0.0f)"),
     "lt":      (2, "(({0} <  {1}) ? 1.0f : 0.0f)"),
@@ -53,16 +56,16 @@ _float_ops = {
     "neg":     (1, "(-{0})"),
     "abs":     (1, "fabsf({0})"),
     "sgn":     (1, "copysignf(1.0f, {0})"),
-    "sqrt":    (1, "sqrtf({0})"),
+    "sqrt":    (1, "__builtin_amdgcn_sqrtf({0})"),
     "sqr":     (1, "({0} * {0})"),
     "exp":     (1, "expf({0})"),
     "log":     (1, "logf({0})"),
     "exp2":    (1, "exp2f({0})"),
     "log2":    (1, "log2f({0})"),
-    "sig":     (1, "(1.0f / (1.0f + expf(-{0})))"),
-    "sig2":    (1, "(1.0f / (1.0f + exp2f(-{0})))"),
+    "sig":     (1, "__builtin_amdgcn_rcpf(1.0f + expf(-{0}))"),
+    "sig2":    (1, "__builtin_amdgcn_rcpf(1.0f + exp2f(-{0}))"),
     "tanh":    (1, "tanhf({0})"),
-    "tanh2":   (1, "((exp2f(2.0f * {0}) - 1.0f) / (exp2f(2.0f * {0}) + 1.0f))"),
+    "tanh2":   (1, "((exp2f(2.0f * {0}) - 1.0f) * __builtin_amdgcn_rcpf(exp2f(2.0f * {0}) + 1.0f))"),
     "rand":    (0, None),
     "onehot":  (0, None),
 }
@@ -585,7 +588,9 @@ def generate_source(spec, name="ew_kernel"):
         if need_idx:
             L.append("            const unsigned rng_idx = (unsigned)row * rng_rm + (unsigned)col * rng_cm; (void)rng_idx;")
         for v in range(V):
-            L.append("            if (col + %d < n) {" % v)
+            # vectors are only used when they divide the row, so a vector that
+            # starts inside the row lies inside it entirely
+            L.append("            {")
             local, blk = {}, []
             for r in stage:
                 val = em.emit_elem(r.args[0], blk, local, "it", str(v)) if not r.args[0].scalar \

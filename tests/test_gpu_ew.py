@@ -59,7 +59,12 @@ def test_math_matrix(ng, dtype):
         inB = np.where(np.abs(inB) < 0.05, dtype(0.5), inB)
         ref = numpy_math("/", inA, inB).astype(dtype)
         got = gpu_math(ng, "/", inA, inB, dtype).get()
-        assert np.array_equal(got, ref), "division must be correctly rounded"
+        # the reference compiles with fast-math division (nervanagpu/float_ew.py:1030);
+        # here x / y is x * rcp(y): within 2 ulp in fp32, then rounded to nearest
+        if dtype is np.float32:
+            np.testing.assert_allclose(got, ref, rtol=2.5e-7, atol=0)
+        else:
+            assert_fp16_within_ulp(got, inA.astype(np.float32) / inB.astype(np.float32), 1, "fp16 division")
 
 
 def test_unary_ops_and_constants(ng):
@@ -67,20 +72,21 @@ def test_unary_ops_and_constants(ng):
     a = rng.uniform(0.1, 2.0, (300, 200)).astype(np.float32)
     A = ng.array(a, dtype=np.float32)
     C = ng.empty(a.shape, dtype=np.float32)
+    # sqrt and division are the hardware approximations (fast-math in the reference)
     cases = [
-        (lambda: ng.sqrt(A), np.sqrt(a), 0), (lambda: ng.square(A), a * a, 0),
+        (lambda: ng.sqrt(A), np.sqrt(a), 2.5e-7), (lambda: ng.square(A), a * a, 0),
         (lambda: ng.exp(A), np.exp(a), 2e-6), (lambda: ng.log(A), np.log(a), 2e-6),
         (lambda: ng.exp2(A), np.exp2(a), 2e-6), (lambda: ng.log2(A), np.log2(a), 2e-6),
         (lambda: ng.sig(A), 1 / (1 + np.exp(-a)), 2e-6), (lambda: ng.tanh(A), np.tanh(a), 2e-6),
         (lambda: ng.tanh2(A), (np.exp2(2 * a) - 1) / (np.exp2(2 * a) + 1), 4e-6),
         (lambda: ng.sig2(A), 1 / (1 + np.exp2(-a)), 2e-6),
-        (lambda: ng.reciprocal(A), (1 / a), 0), (lambda: -A, -a, 0), (lambda: abs(A - 1.0), np.abs(a - np.float32(1)), 0),
+        (lambda: ng.reciprocal(A), (1 / a), 2.5e-7), (lambda: -A, -a, 0), (lambda: abs(A - 1.0), np.abs(a - np.float32(1)), 0),
         (lambda: ng.sgn(A - 1.0), np.copysign(1, a - np.float32(1)), 0),
         (lambda: ng.power(A, 1.5), np.power(a, np.float32(1.5)), 4e-6),
         (lambda: ng.clip(A, 0.5, 1.0), np.clip(a, 0.5, 1.0), 0),
         (lambda: ng.maximum(A, 1.25), np.maximum(a, 1.25), 0), (lambda: ng.minimum(A, 1.25), np.minimum(a, 1.25), 0),
         (lambda: 2.5 * A * A + 1, np.float32(2.5) * a * a + 1, 0),
-        (lambda: 1 - A, 1 - a, 0), (lambda: 2.0 / A, np.float32(2) / a, 0),
+        (lambda: 1 - A, 1 - a, 0), (lambda: 2.0 / A, np.float32(2) / a, 2.5e-7),
         (lambda: (A == A) + (A != A), np.ones_like(a), 0),
         (lambda: ng.finite(ng.log(A - 1.0)), np.isfinite(np.log(a - np.float32(1))).astype(np.float32), 0),
     ]
