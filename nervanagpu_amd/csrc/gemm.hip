@@ -103,12 +103,19 @@ template <typename T> static int dispatch(const GemmArgs& g, unsigned sr_bits);
 template <>
 int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
 {
-    const bool vec = operands_vectorizable<_Float16>(g);
+    if (!operands_vectorizable<_Float16>(g)) return launch_layout<_Float16, 128, 128, 64, 2, 2, false>(g, sr_bits);
+    const int cus = device_cu_count();
+    const int k_tiles = ceil_div(g.k, 64) * g.batch_loops;
+    // 256x256 tiles when they still fill the chip and the contraction is long
+    // enough to amortise their prologue and epilogue
     const long big_tiles = (long)ceil_div(g.m, 256) * ceil_div(g.n, 256) * g.batch_grid;
-    const bool large = g.m >= 256 && g.n >= 256 && big_tiles >= device_cu_count() / 2;
-    if (large && vec) return launch_layout<_Float16, 256, 256, 64, 2, 4, true>(g, sr_bits);
-    return vec ? launch_layout<_Float16, 128, 128, 64, 2, 2, true>(g, sr_bits)
-               : launch_layout<_Float16, 128, 128, 64, 2, 2, false>(g, sr_bits);
+    if (g.m >= 256 && g.n >= 256 && big_tiles >= cus / 2 && k_tiles >= 8)
+        return launch_layout<_Float16, 256, 256, 64, 2, 4, true>(g, sr_bits);
+    // minibatch-wide outputs (n <= 128) stream the weight matrix: halve the row
+    // tile so that fewer contraction slices, i.e. fewer fp32 partials, fill the chip
+    const long tiles128 = (long)ceil_div(g.m, 128) * ceil_div(g.n, 128) * g.batch_grid;
+    if (g.n <= 128 && tiles128 < cus) return launch_layout<_Float16, 64, 128, 64, 2, 2, true>(g, sr_bits);
+    return launch_layout<_Float16, 128, 128, 64, 2, 2, true>(g, sr_bits);
 }
 
 template <>
@@ -153,10 +160,11 @@ size_t ng_gemm_workspace_bytes(int dtype, int trans_a, int trans_b, int m, int n
 {
     (void)trans_a; (void)trans_b;
     const int bk = (dtype == NG_F16) ? 64 : 16;
-    const int bt = 128;
-    const int out_tiles = ceil_div(m, bt) * ceil_div(n, bt) * batch_grid;
     const int total_k = ceil_div(k, bk) * batch_loops;
-    const int splits = choose_splits(out_tiles, total_k, 0, 0);
+    // the largest slice count any tile shape the dispatcher may pick would use
+    int splits = 1;
+    for (int bm : {64, 128})
+        splits = std::max(splits, choose_splits(ceil_div(m, bm) * ceil_div(n, 128) * batch_grid, total_k, 0, 0));
     if (splits <= 1) return 0;
     return (size_t)splits * batch_grid * m * n * sizeof(float);
 }

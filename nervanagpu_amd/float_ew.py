@@ -926,7 +926,7 @@ def analyse(args):
             vec = 1
         plan.vec = vec
         nvec = (max(n, n_out) + vec - 1) // vec
-        threads = min(MAX_THREADS, max(64, _pow2_at_least((nvec + 1) // 2)))
+        threads = min(MAX_THREADS, max(64, _pow2_at_least((nvec + 3) // 4)))
         if not reduction:
             threads = min(threads, 256)
         items = (nvec + threads - 1) // threads
