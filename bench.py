@@ -270,6 +270,26 @@ def format_rows(rows):
     return "\n".join(lines)
 
 
+CAL_COPY_ELEMS = 1 << 27     # fp16 elements of the calibration copy: 256 MiB read + 256 MiB written
+
+
+def calibrate(ng):
+    """Counter calibration run: a flat copy kernel that reads and writes exactly
+    CAL_COPY_ELEMS * 2 bytes, then the 4096^3 fp16 GEMM, five launches each."""
+    from nervanagpu_amd import _lib
+    src = ng.empty((CAL_COPY_ELEMS // 8192, 8192), dtype=np.float16)
+    dst = ng.empty((CAL_COPY_ELEMS // 8192, 8192), dtype=np.float16)
+    src.fill(1.0)
+    for _ in range(5):
+        dst._assign(src)
+    gemm = GemmCase(ng, "nn", 4096, 4096, 4096)
+    for _ in range(5):
+        gemm.run()
+    _lib.stream_sync(ng.stream)
+    print(json.dumps({"calibrate": {"copy_bytes_read": CAL_COPY_ELEMS * 2, "copy_bytes_written": CAL_COPY_ELEMS * 2,
+                                    "gemm": gemm.name()}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -278,6 +298,9 @@ def main():
     ap.add_argument("--all", action="store_true", help="also time every configured case")
     ap.add_argument("--out", default=None, help="file for the --all table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="only launch a plain copy of known size and the dominant GEMM a few times "
+                         "(the run hardware counters are collected on)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (got --gpus %d); "
@@ -285,6 +308,9 @@ def main():
 
     from nervanagpu_amd import NervanaGPU, _lib
     ng = NervanaGPU(stochastic_round=False, bench=False, seed=1)
+    if args.calibrate:
+        calibrate(ng)
+        return
     cases = build_config2(ng)
     step_flops = sum(c.flops for c in cases)
 

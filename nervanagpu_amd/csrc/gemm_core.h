@@ -779,6 +779,21 @@ template <> struct StoreBits<_Float16> {
     {
         return sr_bits ? ng_sr_f16(v, sr_bits, ng_rand_sr16(seed, stream, idx)) : ng_f32_to_f16_rn(v);
     }
+    // random words of 8 consecutive elements starting at an even index: one
+    // draw per pair of elements
+    static __device__ __forceinline__ void words8(unsigned seed, unsigned stream, unsigned idx0, unsigned (&w)[8])
+    {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const unsigned h = ng_rand32(seed, stream, (idx0 >> 1) + k);
+            w[2 * k] = h;
+            w[2 * k + 1] = h << 16;
+        }
+    }
+    static __device__ __forceinline__ bits_t round_word(float v, unsigned sr_bits, unsigned r)
+    {
+        return ng_sr_f16(v, sr_bits, r);
+    }
     static __device__ __forceinline__ float widen(bits_t b) { return ng_f16_to_f32(b); }
 };
 template <> struct StoreBits<float> {
@@ -786,6 +801,15 @@ template <> struct StoreBits<float> {
     static __device__ __forceinline__ bits_t round(float v, unsigned sr_bits, unsigned seed, unsigned stream, unsigned idx)
     {
         return __float_as_uint(sr_bits ? ng_sr_f32(v, sr_bits, ng_rand32(seed, stream, idx)) : v);
+    }
+    static __device__ __forceinline__ void words8(unsigned seed, unsigned stream, unsigned idx0, unsigned (&w)[8])
+    {
+#pragma unroll
+        for (int e = 0; e < 8; e++) w[e] = ng_rand32(seed, stream, idx0 + e);
+    }
+    static __device__ __forceinline__ bits_t round_word(float v, unsigned sr_bits, unsigned r)
+    {
+        return __float_as_uint(ng_sr_f32(v, sr_bits, r));
     }
     static __device__ __forceinline__ float widen(bits_t b) { return __uint_as_float(b); }
 };
@@ -842,12 +866,15 @@ struct ScaleStoreEpilogue {
                 for (int q = 0; q < NV; q++)
                     reinterpret_cast<uint4_t*>(out)[q] = reinterpret_cast<const uint4_t*>(p)[q];
             }
-            const unsigned idx0 = rng_index(i, j0, z);
+            // n and j0 are multiples of 8 here, so the stream index of the first
+            // element is even
+            unsigned words[8];
+            if (sr_bits) StoreBits<T>::words8(seed, stream, rng_index(i, j0, z), words);
 #pragma unroll
             for (int e = 0; e < 8; e++) {
                 float v = scale(acc[e]);
                 if (beta != 0.0f) v += beta * StoreBits<T>::widen(out[e]);
-                out[e] = StoreBits<T>::round(v, sr_bits, seed, stream, idx0 + e);
+                out[e] = sr_bits ? StoreBits<T>::round_word(v, sr_bits, words[e]) : StoreBits<T>::round(v, 0, 0, 0, 0);
             }
 #pragma unroll
             for (int q = 0; q < NV; q++)
@@ -883,15 +910,40 @@ struct PartialEpilogue {
     }
 };
 
-// fixed-order sum of the partial slices followed by the final epilogue
+// fixed-order sum of the partial slices followed by the final epilogue.
+// vec8: n is a multiple of 8; a thread then owns 8 consecutive columns of a row
+// (32-byte loads from every slice, one 16-byte store).
 template <typename T, class Epi>
-__global__ void splitk_reduce_kernel(const float* ws, int splits, int zcount, int m, int n, Epi epi)
+__global__ __launch_bounds__(256)
+void splitk_reduce_kernel(const float* __restrict__ ws, int splits, int zcount, int m, int n, Epi epi, unsigned vec8)
 {
     const long total = (long)zcount * m * n;
-    const long slice = total;
-    for (long e = (long)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (long)gridDim.x * blockDim.x) {
+    if (vec8) {
+        const long groups = total >> 3;
+        const int per_row = n >> 3;
+        for (long g = (long)blockIdx.x * 256 + threadIdx.x; g < groups; g += (long)gridDim.x * 256) {
+            float acc[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[e] = 0.0f;
+            const float* p = ws + g * 8;
+#pragma unroll 4
+            for (int sidx = 0; sidx < splits; sidx++) {
+                const float4_t lo = *reinterpret_cast<const float4_t*>(p + sidx * total);
+                const float4_t hi = *reinterpret_cast<const float4_t*>(p + sidx * total + 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) { acc[e] += lo[e]; acc[e + 4] += hi[e]; }
+            }
+            const long r = g / per_row;
+            const int j0 = (int)(g - r * per_row) * 8;
+            const int i = (int)(r % m);
+            const int z = (int)(r / m);
+            epi.store8(i, j0, z, 0, acc);
+        }
+        return;
+    }
+    for (long e = (long)blockIdx.x * 256 + threadIdx.x; e < total; e += (long)gridDim.x * 256) {
         float acc = 0.0f;
-        for (int sidx = 0; sidx < splits; sidx++) acc += ws[sidx * slice + e];
+        for (int sidx = 0; sidx < splits; sidx++) acc += ws[sidx * total + e];
         const int j = (int)(e % n);
         const long r = e / n;
         const int i = (int)(r % m);
