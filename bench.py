@@ -270,6 +270,11 @@ def format_rows(rows):
     return "\n".join(lines)
 
 
+# HBM bytes per launch of the 4096^3 kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on
+# `bench.py --calibrate`, each scaled by the same counter's reading for the 256 MiB copy
+# (147700 KiB x 2.0 fetched + 32768 KiB x 1.0 written); algorithmic bytes are 100.7e6
+DOMINANT_TRAFFIC_BYTES = 336.0e6
+
 CAL_COPY_ELEMS = 1 << 27     # fp16 elements of the calibration copy: 256 MiB read + 256 MiB written
 
 
@@ -331,9 +336,9 @@ def main():
     dominant = [c for c in cases if c.m == c.n == c.k == 4096][0]
     dom_ms = time_gpu(ng, dominant.run, iters=max(args.steps, 20), warmup=3)
     achieved = dominant.flops / dom_ms / 1e9
-    roofline = {"bound": "mfma", "kernel": "mfma_gemm_kernel<fp16,256x256x32,nn> (4096^3)",
+    roofline = {"bound": "mfma", "kernel": "mfma_gemm_direct_kernel<fp16,256x256x64,A:KC,B:MC,2 stages> (4096^3 nn)",
                 "achieved": achieved, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                "frac": achieved / PEAK_FP16_TFLOPS, "traffic": None,
+                "frac": achieved / PEAK_FP16_TFLOPS, "traffic": DOMINANT_TRAFFIC_BYTES,
                 "launch_ms": dom_ms, "flops_per_launch": dominant.flops}
 
     result = {
