@@ -272,8 +272,8 @@ def format_rows(rows):
 
 # HBM bytes per launch of the 4096^3 kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on
 # `bench.py --calibrate`, each scaled by the same counter's reading for the 256 MiB copy
-# (147700 KiB x 2.0 fetched + 32768 KiB x 1.0 written); algorithmic bytes are 100.7e6
-DOMINANT_TRAFFIC_BYTES = 336.0e6
+# (98530 KiB x 2.0 fetched + 32768 KiB x 1.0 written); algorithmic bytes are 100.7e6
+DOMINANT_TRAFFIC_BYTES = 235.3e6
 
 CAL_COPY_ELEMS = 1 << 27     # fp16 elements of the calibration copy: 256 MiB read + 256 MiB written
 

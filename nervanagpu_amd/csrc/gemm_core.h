@@ -236,15 +236,23 @@ struct DenseLoader {
 };
 
 // blockIdx.x -> (tile_m, tile_n).  Workgroups are handed to the 8 XCDs round
-// robin; renumbering them so that each XCD works on a contiguous range of tiles
-// keeps the operand tiles it re-reads in its own L2.
+// robin; renumbering them gives each XCD a contiguous range of tile numbers,
+// and numbering the tiles in bands of 8 rows (column-major inside a band) makes
+// such a range a compact block of the output (e.g. 8 x 4 tiles for 32 CUs
+// instead of 16 x 2), so fewer distinct operand tiles pass through its L2.
 __device__ __forceinline__ void tile_of_block(const CoreShape& s, int& tm, int& tn)
 {
     int pid = blockIdx.x;
     const int total = gridDim.x;
     if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
-    tm = pid % s.tiles_m;
-    tn = pid / s.tiles_m;
+    constexpr int BAND = 8;
+    const int per_band = BAND * s.tiles_n;
+    const int band = pid / per_band;
+    const int first_m = band * BAND;
+    const int rows = min(BAND, s.tiles_m - first_m);
+    const int in_band = pid - band * per_band;
+    tn = in_band / rows;
+    tm = first_m + (in_band - tn * rows);
 }
 
 // Scheduling directive for one k-step.  After each MFMA: two LDS reads of the
