@@ -410,7 +410,7 @@ def generate_source(spec, name="ew_kernel"):
                 else:
                     idx = "(long)(%s + %d) * cs%d" % (base_col, v, arg_id)
                 rid = "rng_idx + %du" % v if not rng_strided else "rng_idx + %du * rng_cm" % v
-                o.append("%sif (%s + %d < n_out) p%d[%s] = %s;" % (pad, base_col, v, arg_id, idx, _gen_round(code, vals[v], rounding, rid)))
+                o.append("%sif (active && %s + %d < n_out) p%d[%s] = %s;" % (pad, base_col, v, arg_id, idx, _gen_round(code, vals[v], rounding, rid)))
         return o
 
     uses_rand = any(a[0] == "rand" for a in spec.type_args)
@@ -469,13 +469,27 @@ def generate_source(spec, name="ew_kernel"):
         return "\n".join(L), args
 
     # ---------------- row mode ----------------
+    # "row": a workgroup owns one row, lanes walk along it.
+    # "col": rows are unit-stride neighbours in memory (a reduction down the
+    #        columns of a row-major matrix): a workgroup owns 64 adjacent rows,
+    #        one per lane, so every wavefront load is one contiguous run; the
+    #        wavefronts of the workgroup split the reduction axis and combine in LDS.
+    col_mode = spec.mode == "col"
     rng_strided = True
     L.append("    const int lane = tid & 63, wave = tid >> 6;")
-    L.append("    const long row = blockIdx.x;")
-    L.append("    if (row >= rows) return;")
-    L.append("    __shared__ float red_f[THREADS / 64 + 1];")
-    L.append("    __shared__ int red_i[THREADS / 64 + 1];")
-    L.append("    (void)lane; (void)wave; (void)red_f; (void)red_i;")
+    if col_mode:
+        L.append("    const long row_raw = (long)blockIdx.x * 64 + lane;")
+        L.append("    const bool active = row_raw < rows;")
+        L.append("    const long row = active ? row_raw : rows - 1;")
+        L.append("    __shared__ float red_f[THREADS];")
+        L.append("    __shared__ int red_i[THREADS];")
+    else:
+        L.append("    const long row = blockIdx.x;")
+        L.append("    if (row >= rows) return;")
+        L.append("    const bool active = true;")
+        L.append("    __shared__ float red_f[THREADS / 64 + 1];")
+        L.append("    __shared__ int red_i[THREADS / 64 + 1];")
+    L.append("    (void)lane; (void)wave; (void)red_f; (void)red_i; (void)active;")
     for t in spec.tensors:
         arg_id, code, access, take_axis, is_out = t
         if take_axis == 1:
@@ -492,6 +506,12 @@ def generate_source(spec, name="ew_kernel"):
     loaded = set()
 
     def loop_open(bound):
+        if col_mode:
+            if ITEMS:
+                return ["    _Pragma(\"unroll\") for (int it = 0; it < %d; it++) {" % ITEMS,
+                        "        const int col = it * (THREADS / 64) + wave;",
+                        "        if (col < %s) {" % bound]
+            return ["    _Pragma(\"unroll 8\") for (int col = wave; col < %s; col += THREADS / 64) {" % bound, "        {"]
         if ITEMS:
             return ["    _Pragma(\"unroll\") for (int it = 0; it < %d; it++) {" % ITEMS,
                     "        const int col = (it * THREADS + tid) * VEC;",
@@ -536,6 +556,23 @@ def generate_source(spec, name="ew_kernel"):
     def block_reduce(kind, var, ivar=None):
         o = []
         comb = {"sum": "{0} += {1};", "max": "{0} = fmaxf({0}, {1});", "min": "{0} = fminf({0}, {1});"}
+        if col_mode:
+            # lanes are different rows: combine the wavefronts' partials only
+            if T == 64:
+                return o
+            if kind in comb:
+                o.append("    __syncthreads(); red_f[tid] = %s; __syncthreads();" % var)
+                o.append("    %s = red_f[lane];" % var)
+                o.append("    _Pragma(\"unroll\") for (int w = 1; w < THREADS / 64; w++) { const float o_ = red_f[w * 64 + lane]; %s }"
+                         % comb[kind].format(var, "o_"))
+            else:
+                better = ">" if kind == "argmax" else "<"
+                merge = ("if (o_ %s %s || (o_ == %s && oi_ >= 0 && (oi_ < %s || %s < 0))) { %s = o_; %s = oi_; }"
+                         % (better, var, var, ivar, ivar, var, ivar))
+                o.append("    __syncthreads(); red_f[tid] = %s; red_i[tid] = %s; __syncthreads();" % (var, ivar))
+                o.append("    %s = red_f[lane]; %s = red_i[lane];" % (var, ivar))
+                o.append("    _Pragma(\"unroll\") for (int w = 1; w < THREADS / 64; w++) { const float o_ = red_f[w * 64 + lane]; const int oi_ = red_i[w * 64 + lane]; %s }" % merge)
+            return o
         if kind in comb:
             o.append("    _Pragma(\"unroll\") for (int off = 32; off > 0; off >>= 1) { const float o_ = __shfl_xor(%s, off, 64); %s }"
                      % (var, comb[kind].format(var, "o_")))
@@ -628,7 +665,7 @@ def generate_source(spec, name="ew_kernel"):
     if red_out:
         val = em.emit_scalar_tree(root, L)
         arg_id, code = out_t[0], out_t[1]
-        L.append("    if (tid == 0) {")
+        L.append("    if (%s) {" % ("wave == 0 && active" if col_mode else "tid == 0"))
         L.append("        const unsigned rng_idx = (unsigned)row * rng_rm; (void)rng_idx;")
         L.append("        p%d[0] = %s;" % (arg_id, _gen_round(code, val, rounding, "rng_idx")))
         L.append("    }")
@@ -926,15 +963,28 @@ def analyse(args):
             vec = 1
         plan.vec = vec
         nvec = (max(n, n_out) + vec - 1) // vec
-        threads = min(MAX_THREADS, max(64, _pow2_at_least((nvec + 3) // 4)))
-        if not reduction:
-            threads = min(threads, 256)
-        items = (nvec + threads - 1) // threads
+        streamed = [v for v in values.values() if "ptr" in v and (v["cs"] != 0 or v["is_out"])]
+        col_mode = (vec == 1 and rows >= 32 and not any(v["take_axis"] for v in values.values() if "ptr" in v)
+                    and all(v["rs"] in (0, 1) for v in values.values() if "ptr" in v)
+                    and any(v["rs"] == 1 for v in streamed))
+        if col_mode:
+            # neighbouring rows are adjacent in memory: one row per lane, the
+            # wavefronts of a workgroup share the walk along the row
+            plan.mode = "col"
+            groups = min(16, max(1, _pow2_at_least((nvec + 7) // 8)))
+            threads = 64 * groups
+            items = (nvec + groups - 1) // groups
+            plan.grid = (rows + 63) // 64
+        else:
+            threads = min(MAX_THREADS, max(64, _pow2_at_least((nvec + 3) // 4)))
+            if not reduction:
+                threads = min(threads, 256)
+            items = (nvec + threads - 1) // threads
+            plan.grid = rows
         # keep the row in registers only when every loop walks the same extent
         if items * vec > MAX_CACHED_PER_LANE or not reduction or n_out not in (1, n):
             items = 0
         plan.threads, plan.items = threads, items
-        plan.grid = rows
         tensors = []
         for i, v in sorted(values.items()):
             if "ptr" not in v:
