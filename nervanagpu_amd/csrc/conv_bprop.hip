@@ -54,8 +54,7 @@ template <bool BLOCKED>
 static int bprop_class_h(const ConvPlan& pl, const BpropClass& c, const _Float16* Fs, const void* E, void* gradI,
                          float alpha, hipStream_t st)
 {
-    static const int tiles[3] = {256, 128, 64};
-    switch (pick_row_tile(pl.p.C, tiles, 3)) {
+    switch (pick_row_tile(pl.p.C, c.nz * c.ny * c.nx * pl.p.N, 256)) {
     case 256: return bprop_class<_Float16, BLOCKED, 256, 256, 64, 2, 4>(pl, c, Fs, E, gradI, alpha, st);
     case 128: return bprop_class<_Float16, BLOCKED, 128, 256, 64, 1, 4>(pl, c, Fs, E, gradI, alpha, st);
     default:  return bprop_class<_Float16, BLOCKED, 64, 256, 64, 1, 4>(pl, c, Fs, E, gradI, alpha, st);

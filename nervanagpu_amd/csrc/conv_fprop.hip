@@ -33,8 +33,7 @@ static int fprop_tile(const ConvPlan& pl, const void* I, const void* F, void* O,
 template <typename TIN, bool BLOCKED>
 static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags, hipStream_t st)
 {
-    static const int tiles[3] = {256, 128, 64};
-    switch (pick_row_tile(pl.p.K, tiles, 3)) {
+    switch (pick_row_tile(pl.p.K, pl.p.M * pl.p.P * pl.p.Q * pl.p.N, 256)) {
     case 256: return fprop_tile<_Float16, TIN, BLOCKED, 256, 256, 64, 2, 4>(pl, I, F, O, alpha, flags, st);
     case 128: return fprop_tile<_Float16, TIN, BLOCKED, 128, 256, 64, 1, 4>(pl, I, F, O, alpha, flags, st);
     default:  return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 64, 1, 4>(pl, I, F, O, alpha, flags, st);

@@ -54,13 +54,22 @@ inline int check_ptr16(const void* p, const char* what)
     return 0;
 }
 
-// row tile (output feature maps or input channels) with the least padding
-inline int pick_row_tile(int rows, const int* tiles, int n)
+// Row tile (output feature maps or input channels) for BN-column tiles: the
+// candidate with the least estimated time, rounds of workgroups over the chip
+// times the work of one workgroup, where the 256-row tile runs about a third
+// more efficiently than the narrower ones (measured on dense problems).
+// Padding rows count as work, so a 64-row problem picks the 64-row tile.
+inline int pick_row_tile(int rows, int ncols, int bn)
 {
-    int best = tiles[0], best_pad = cdiv(rows, best) * best;
-    for (int i = 1; i < n; i++) {
-        const int pad = cdiv(rows, tiles[i]) * tiles[i];
-        if (pad < best_pad) { best = tiles[i]; best_pad = pad; }
+    static const int tiles[3] = {256, 128, 64};
+    static const double eff[3] = {1.0, 0.75, 0.75};
+    const int cus = device_cu_count();
+    int best = tiles[0];
+    double best_cost = 0.0;
+    for (int i = 0; i < 3; i++) {
+        const long blocks = (long)cdiv(rows, tiles[i]) * cdiv(ncols, bn);
+        const double cost = (double)((blocks + cus - 1) / cus) * tiles[i] / eff[i];
+        if (i == 0 || cost < best_cost * 0.999) { best = tiles[i]; best_cost = cost; }
     }
     return best;
 }

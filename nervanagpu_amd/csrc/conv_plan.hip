@@ -99,8 +99,9 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
     pl->ws_bprop = align_up((size_t)pl->RST * p.K * pl->Cpad * dtype_size(dtype), 256);
     {
         const int kt = cdiv(p.M * p.P * p.Q * p.N, pl->bk);
-        const int tiles = cdiv(pl->CRST, 128) * cdiv(p.K, 128);
-        const int splits = conv_splits(tiles, kt, 0, 0);
+        // the most slices any tile shape of the update dispatcher would ask for
+        const int splits = std::max(conv_splits(cdiv(pl->CRST, 128) * cdiv(p.K, 128), kt, 0, 0),
+                                    conv_splits(cdiv(pl->CRST, 256) * cdiv(p.K, 256), kt, 0, 0));
         pl->ws_update = splits > 1 ? align_up((size_t)splits * pl->CRST * p.K * sizeof(float), 256) : 0;
     }
     *plan_out = pl;

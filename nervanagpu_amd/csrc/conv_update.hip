@@ -46,8 +46,18 @@ template <typename TIN, typename TOUT>
 static int update_h(const ConvPlan& pl, const void* I, const void* E, void* gradF, float alpha,
                     void* ws, size_t ws_bytes, hipStream_t st)
 {
-    if (pl.p.N % 64 == 0)
+    if (pl.p.N % 64 == 0) {
+        // fp16 activations: tile shaped after the filter matrix (CRST x K)
+        if constexpr (std::is_same<TIN, _Float16>::value) {
+            // 256x256 tiles leave few output tiles, i.e. many contraction slices
+            // and fp32 partials: worth it only for long pixel ranges
+            if (pl.p.K >= 256 && pl.CRST >= 256 && (long)pl.p.M * pl.p.P * pl.p.Q * pl.p.N >= 512 * 64)
+                return launch_update<_Float16, TIN, TOUT, true, 256, 256, 64, 2, 4>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
+            if (pl.p.K <= 64)
+                return launch_update<_Float16, TIN, TOUT, true, 128, 64, 64, 2, 2>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
+        }
         return launch_update<_Float16, TIN, TOUT, true, 128, 128, 64, 2, 2>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
+    }
     return launch_update<_Float16, TIN, TOUT, false, 128, 128, 64, 2, 2>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
 }
 
