@@ -38,7 +38,7 @@ static int choose_splits(int out_tiles, int total_k_tiles, size_t slice_bytes, s
     return std::max(splits, 1);
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, bool VEC>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, bool VEC, int NSTAGE = 2>
 static int launch_gemm(const GemmArgs& g, unsigned sr_bits)
 {
     CoreShape s;
@@ -60,11 +60,11 @@ static int launch_gemm(const GemmArgs& g, unsigned sr_bits)
 
     dim3 grid(s.tiles_m * s.tiles_n, s.splits, zcount);
     if (s.splits == 1) {
-        launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB>(grid, g.stream, al, bl, epi, s);
+        launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB, NSTAGE>(grid, g.stream, al, bl, epi, s);
         NG_CHECK_LAUNCH("gemm kernel");
     } else {
         PartialEpilogue pe{(float*)g.ws, g.m, g.n, zcount, (g.n % 8 == 0) ? 1u : 0u};
-        launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB>(grid, g.stream, al, bl, pe, s);
+        launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB, NSTAGE>(grid, g.stream, al, bl, pe, s);
         NG_CHECK_LAUNCH("gemm split kernel");
         const long total = (long)zcount * g.m * g.n;
         const unsigned vec8 = (g.n % 8 == 0) ? 1u : 0u;
@@ -77,12 +77,12 @@ static int launch_gemm(const GemmArgs& g, unsigned sr_bits)
     return 0;
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, bool VEC>
+template <typename T, int BM, int BN, int BK, int WM, int WN, bool VEC, int NSTAGE = 2>
 static int launch_layout(const GemmArgs& g, unsigned sr_bits)
 {
-    if (!g.trans_a && !g.trans_b) return launch_gemm<T, BM, BN, BK, WM, WN, KC, MC, VEC>(g, sr_bits);
-    if (!g.trans_a && g.trans_b)  return launch_gemm<T, BM, BN, BK, WM, WN, KC, KC, VEC>(g, sr_bits);
-    return launch_gemm<T, BM, BN, BK, WM, WN, MC, MC, VEC>(g, sr_bits);
+    if (!g.trans_a && !g.trans_b) return launch_gemm<T, BM, BN, BK, WM, WN, KC, MC, VEC, NSTAGE>(g, sr_bits);
+    if (!g.trans_a && g.trans_b)  return launch_gemm<T, BM, BN, BK, WM, WN, KC, KC, VEC, NSTAGE>(g, sr_bits);
+    return launch_gemm<T, BM, BN, BK, WM, WN, MC, MC, VEC, NSTAGE>(g, sr_bits);
 }
 
 template <typename T>
@@ -116,8 +116,11 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
     // minibatch-wide outputs (n <= 128) stream the weight matrix: halve the row
     // tile so that fewer contraction slices, i.e. fewer fp32 partials, fill the chip
     const long tiles128 = (long)ceil_div(g.m, 128) * ceil_div(g.n, 128) * g.batch_grid;
-    if (g.n <= 128 && tiles128 < cus) return launch_layout<_Float16, 64, 128, 64, 2, 2, true>(g, sr_bits);
-    return launch_layout<_Float16, 128, 128, 64, 2, 2, true>(g, sr_bits);
+    if (tiles128 >= cus) return launch_layout<_Float16, 128, 128, 64, 2, 2, true>(g, sr_bits);
+    if (g.n <= 128) return launch_layout<_Float16, 64, 128, 64, 2, 2, true>(g, sr_bits);
+    // mid-sized outputs: small tiles fill the chip without (or with fewer)
+    // contraction slices, which cost fp32 partials and a second launch
+    return launch_layout<_Float16, 64, 64, 64, 2, 2, true>(g, sr_bits);
 }
 
 template <>
@@ -166,7 +169,8 @@ size_t ng_gemm_workspace_bytes(int dtype, int trans_a, int trans_b, int m, int n
     // the largest slice count any tile shape the dispatcher may pick would use
     int splits = 1;
     for (int bm : {64, 128})
-        splits = std::max(splits, choose_splits(ceil_div(m, bm) * ceil_div(n, 128) * batch_grid, total_k, 0, 0));
+        for (int bn : {64, 128})
+            splits = std::max(splits, choose_splits(ceil_div(m, bm) * ceil_div(n, bn) * batch_grid, total_k, 0, 0));
     if (splits <= 1) return 0;
     return (size_t)splits * batch_grid * m * n * sizeof(float);
 }

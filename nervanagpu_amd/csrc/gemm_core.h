@@ -963,12 +963,13 @@ void splitk_reduce_kernel(const float* __restrict__ ws, int splits, int zcount, 
 // Launch the contraction core: the direct-to-LDS pipeline when both operands
 // are plain 16-byte buffer loads of 16-bit elements, the register-staged one
 // otherwise (fp32, element-wise edge handling, 8-bit inputs converted on load).
-template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, class ALoad, class BLoad, class Epi>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, int NSTAGE = 2, class ALoad, class BLoad,
+          class Epi>
 inline void launch_mfma_core(dim3 grid, hipStream_t stream, const ALoad& al, const BLoad& bl, const Epi& epi,
                              const CoreShape& s)
 {
     if constexpr (sizeof(T) == 2 && ALoad::DIRECT && BLoad::DIRECT) {
-        hipLaunchKernelGGL((mfma_gemm_direct_kernel<T, BM, BN, BK, WM, WN, LA, LB, 2, ALoad, BLoad, Epi>), grid,
+        hipLaunchKernelGGL((mfma_gemm_direct_kernel<T, BM, BN, BK, WM, WN, LA, LB, NSTAGE, ALoad, BLoad, Epi>), grid,
                            dim3(WM * WN * 64), 0, stream, al, bl, epi, s);
     } else {
         hipLaunchKernelGGL((mfma_gemm_kernel<T, BM, BN, BK, WM, WN, LA, LB, ALoad, BLoad, Epi>), grid,
