@@ -126,9 +126,10 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
 template <>
 int dispatch<float>(const GemmArgs& g, unsigned sr_bits)
 {
-    const bool vec = operands_vectorizable<float>(g);
-    return vec ? launch_layout<float, 128, 128, 16, 2, 2, true>(g, sr_bits)
-               : launch_layout<float, 128, 128, 16, 2, 2, false>(g, sr_bits);
+    if (!operands_vectorizable<float>(g)) return launch_layout<float, 128, 128, 16, 2, 2, false>(g, sr_bits);
+    const long tiles128 = (long)ceil_div(g.m, 128) * ceil_div(g.n, 128) * g.batch_grid;
+    if (tiles128 >= device_cu_count() || g.n <= 128) return launch_layout<float, 128, 128, 16, 2, 2, true>(g, sr_bits);
+    return launch_layout<float, 64, 64, 32, 2, 2, true>(g, sr_bits);
 }
 
 static int check_args(const GemmArgs& g, int dtype)
