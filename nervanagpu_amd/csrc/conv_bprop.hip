@@ -32,7 +32,7 @@ static int bprop_class(const ConvPlan& pl, const BpropClass& c, const T* Fs, con
     const ng_conv_params& p = pl.p;
     const int ncols = c.nz * c.ny * c.nx * p.N;
     const int MPQN = p.M * p.P * p.Q * p.N;
-    PixelLattice lat{p.N, ncols, c.nx, c.nx * c.ny};
+    const PixelLattice lat = PixelLattice::make(p.N, ncols, c.nx, c.nx * c.ny);
     DenseLoader<T, MC, true> al{Fs + c.w_row * pl.Cpad, 0, pl.Cpad, pl.Cpad, c.J};
     const int nblk = BLOCKED ? p.K / BK : 1;
     GatherColsLoader<T, T, BLOCKED, BK> bl{(const T*)E,

@@ -13,7 +13,7 @@ static int fprop_tile(const ConvPlan& pl, const void* I, const void* F, void* O,
     const int DHWN = p.D * p.H * p.W * p.N;
     ScaleStoreEpilogue<T> epi{(T*)O, 0, ncols, p.K, ncols, alpha, 0.0f,
                               (flags & NG_FLAG_RELU) ? 1u : 0u, 0u, 0u, 0u, 1u};
-    PixelLattice lat{p.N, ncols, p.Q, p.P * p.Q};
+    const PixelLattice lat = PixelLattice::make(p.N, ncols, p.Q, p.P * p.Q);
     if (BLOCKED) {
         const int nblk = p.C / BK;
         FilterBlockLoader<T, BK> al{(const T*)F, p.K, pl.RST * p.K, FastDiv::make((unsigned)nblk), nblk};

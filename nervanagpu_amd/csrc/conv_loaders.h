@@ -84,6 +84,23 @@ struct PixelLattice {
     int N;
     int ncols;      // nz*ny*nx*N
     int nx, nxy;    // nx, nx*ny
+    FastDiv div_n, div_nxy, div_nx;
+
+    static PixelLattice make(int N, int ncols, int nx, int nxy)
+    {
+        return PixelLattice{N, ncols, nx, nxy, FastDiv::make((unsigned)N), FastDiv::make((unsigned)nxy),
+                            FastDiv::make((unsigned)nx)};
+    }
+    // column -> (iz, iy, ix, n)
+    __device__ __forceinline__ void split(int col, int& iz, int& iy, int& ix, int& nn) const
+    {
+        const int pix = (int)div_n.div((unsigned)col);
+        nn = col - pix * N;
+        iz = (int)div_nxy.div((unsigned)pix);
+        const int rem = pix - iz * nxy;
+        iy = (int)div_nx.div((unsigned)rem);
+        ix = rem - iy * nx;
+    }
 };
 
 #define NG_FAR (-0x40000000)
@@ -115,9 +132,8 @@ struct GatherColsLoader {
         Ctx c;
         c.kr = kr;
         if (col >= lat.ncols) { c.base = 0; c.z0 = c.y0 = c.x0 = NG_FAR; return c; }
-        const int pix = col / lat.N, nn = col - pix * lat.N;
-        const int iz = pix / lat.nxy, rem = pix - iz * lat.nxy;
-        const int iy = rem / lat.nx, ix = rem - iy * lat.nx;
+        int iz, iy, ix, nn;
+        lat.split(col, iz, iy, ix, nn);
         c.z0 = iz * gs_d; c.y0 = iy * gs_h; c.x0 = ix * gs_w;
         c.base = ((c.z0 * lim_h + c.y0) * lim_w + c.x0) * lat.N + nn;
         if (BLOCKED) c.base += kr * row_stride;
@@ -293,9 +309,8 @@ struct LatticeStoreEpilogue {
     __device__ __forceinline__ void store8(int i, int j0, int /*z*/, int /*split*/, const float (&acc)[8]) const
     {
         if (i >= rows || j0 >= lat.ncols) return;
-        const int pix = j0 / lat.N, nn = j0 - pix * lat.N;
-        const int iz = pix / lat.nxy, rem = pix - iz * lat.nxy;
-        const int iy = rem / lat.nx, ix = rem - iy * lat.nx;
+        int iz, iy, ix, nn;
+        lat.split(j0, iz, iy, ix, nn);
         bits_t* p = reinterpret_cast<bits_t*>(
             out + i * row_stride + (long)(((oz + sz * iz) * H + (oy + sy * iy)) * W + (ox + sx * ix)) * lat.N + nn);
         bits_t b[8];
