@@ -123,6 +123,7 @@ struct GatherColsLoader {
 
     // same-type inputs are plain 16-byte buffer loads (see DenseLoader::DIRECT)
     static constexpr bool DIRECT = std::is_same<T, TIN>::value;
+    static constexpr bool TILE_READS_TABLE = BLOCKED;
 
     struct Ctx { int base, z0, y0, x0, kr; };
     struct Tile { BufferRsrc rsrc; int toff, dz, dy, dx, k0; };
@@ -192,6 +193,7 @@ struct FilterBlockLoader {
     int      nblk;
 
     static constexpr bool DIRECT = true;
+    static constexpr bool TILE_READS_TABLE = false;
 
     struct Ctx { unsigned off; };
     struct Tile { BufferRsrc rsrc; };
@@ -230,6 +232,7 @@ struct GatherRowsLoader {
     int             npt;
 
     static constexpr bool DIRECT = std::is_same<T, TIN>::value;
+    static constexpr bool TILE_READS_TABLE = false;
 
     struct Ctx { int off, dz, dy, dx, kc; };
     struct Tile { BufferRsrc rsrc; int pixbase, z0, y0, x0, k0; };

@@ -184,6 +184,7 @@ struct DenseLoader {
     // a chunk is one 16-byte buffer load whose offset offset() returns, so the
     // core may send it straight to LDS
     static constexpr bool DIRECT = VEC;
+    static constexpr bool TILE_READS_TABLE = false;
 
     struct Ctx { unsigned off; int k; int r; };
     struct Tile { BufferRsrc rsrc; const T* p; int krem; };
@@ -671,11 +672,25 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     constexpr int N_CHUNKS = CPT_A + CPT_B;
     typename ALoad::Tile g_ta;
     typename BLoad::Tile g_tb;
+    // Tile descriptors (they may involve scalar table loads) are prepared one
+    // request ahead when that is free.  Not for the 8-wavefront shapes, which
+    // have no registers to spare, and not when a descriptor reads a table: a
+    // scalar load in flight makes every later LDS wait a full wait
+    // (scalar and LDS operations share one counter and return out of order).
+    constexpr bool PREP_AHEAD = NT <= 256 && !ALoad::TILE_READS_TABLE && !BLoad::TILE_READS_TABLE;
+    int g_left = ntiles;
+    auto gprep = [&]() {
+        if (g_left > 0) {
+            g_ta = aload.tile(g_kt, g_kt * BK, z + g_pass);
+            g_tb = bload.tile(g_kt, g_kt * BK, z + g_pass);
+            if (++g_kt == s.k_tiles) { g_kt = 0; g_pass++; }
+            g_left--;
+        }
+    };
+    if (PREP_AHEAD) gprep();
     // fetch the next global tile into the LDS stage at byte offset `stage_off`
     auto gissue = [&](int stage_off) {
-        g_ta = aload.tile(g_kt, g_kt * BK, z + g_pass);
-        g_tb = bload.tile(g_kt, g_kt * BK, z + g_pass);
-        if (++g_kt == s.k_tiles) { g_kt = 0; g_pass++; }
+        if (!PREP_AHEAD) gprep();
 #pragma unroll
         for (int i = 0; i < CPT_A; i++)
             buffer_load_chunk_to_lds(g_ta.rsrc, smem + stage_off + (i * NT + wave * 64) * 16, aload.offset(g_ta, actx[i]));
@@ -683,6 +698,7 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
         for (int i = 0; i < CPT_B; i++)
             buffer_load_chunk_to_lds(g_tb.rsrc, smem + stage_off + TA::BYTES + (i * NT + wave * 64) * 16,
                                      bload.offset(g_tb, bctx[i]));
+        if (PREP_AHEAD) gprep();
     };
 
     // lane-constant fragment addresses
