@@ -1004,10 +1004,17 @@ def analyse(args):
     return plan
 
 
+_GPUTensor = None
+
+
 def _signature(args):
     """Everything about a postfix stack that the analysis depends on, leaving out
     what is merely passed through to the kernel (addresses, constant values)."""
-    from .nervanagpu import GPUTensor
+    global _GPUTensor
+    if _GPUTensor is None:
+        from .nervanagpu import GPUTensor as _T
+        _GPUTensor = _T
+    GPUTensor = _GPUTensor
     sig = []
     tensors, consts = {}, {}
     for arg in args:

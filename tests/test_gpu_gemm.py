@@ -54,6 +54,25 @@ def test_dot_odd_sizes(ng, dtype, op):
                acc_atol(_absdot(A, B)))
 
 
+# 16-byte aligned operands whose extents are not multiples of any tile: one
+# shape per tile shape of the dispatcher (64x64, 64x128, 128x128, 256x256),
+# so the direct-to-LDS pipeline meets ragged edges in m, n and k
+ALIGNED_RAGGED = [(1000, 136, 520), (520, 128, 1032), (1032, 1000, 72), (2056, 2040, 136), (3080, 3080, 520),
+                  (8, 8, 8), (72, 4104, 264)]
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("op", ["nn", "nt", "tn"])
+def test_dot_aligned_ragged_edges(ng, dtype, op):
+    rng = np.random.default_rng(12)
+    for (m, n, k) in ALIGNED_RAGGED:
+        A, B, dA, dB = _operands(ng, op, m, n, k, dtype, rng)
+        C = ng.empty((m, n), dtype=dtype)
+        ng.dot(dA, dB, C)
+        _check(C.get(), orc.ref_dot(A, B), dtype, "%s %s m,n,k=%d,%d,%d" % (np.dtype(dtype), op, m, n, k),
+               acc_atol(_absdot(A, B)))
+
+
 @pytest.mark.parametrize("op", ["nn", "tn"])
 def test_config1_fp32_1024(ng, op):
     rng = np.random.default_rng(0)
