@@ -4,8 +4,12 @@
 //
 // Always the gather form, for every C and stride: strided layers are decomposed
 // into str_d*str_h*str_w stride-1 sub-problems (one per residue class of the
-// input pixel), each with only the taps that can reach that class.  No atomics,
-// no zero fill, fp32 accumulation, one rounding.
+// input pixel), each with only the taps that can reach that class.  When all
+// classes together have at most 256 rows (few channels, e.g. a first layer)
+// they are stacked into ONE problem: the output-pixel offsets a lattice point
+// reads are the same for every class, so the gathered operand is shared and E
+// is read once instead of once per class.  No atomics, no zero fill, fp32
+// accumulation, one rounding.
 #include "conv_plan.h"
 
 namespace ng {
@@ -22,6 +26,76 @@ __global__ void filter_relayout_kernel(const T* F, T* out, const int* tap_dest, 
         const int trs = (int)(r / K);
         const T v = (c < C) ? F[((long)c * RST + trs) * K + k] : (T)0;
         out[((long)tap_dest[trs] + k) * Cpad + c] = v;
+    }
+}
+
+// filter (C,TRS,K) -> merged matrix [(offset,k)][rpad], rows (class, c): the
+// tap of class (rz,ry,rx) that reads output offset (dz,dy,dx) is
+// (rz + pad_d - dz*str_d, ...); rows whose tap falls outside the filter are zero
+template <typename T>
+__global__ void filter_merge_kernel(const T* F, T* out, const TapEntry* mtaps, ng_conv_params p, int m_taps,
+                                    int m_rows, int m_rpad)
+{
+    const long total = (long)m_taps * p.K * m_rpad;
+    const int RST = p.T * p.R * p.S;
+    for (long e = (long)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (long)gridDim.x * blockDim.x) {
+        const int row = (int)(e % m_rpad);
+        const long r = e / m_rpad;
+        const int k = (int)(r % p.K);
+        const int mt = (int)(r / p.K);
+        T v = (T)0;
+        if (row < m_rows) {
+            const int cls = row / p.C, c = row - cls * p.C;
+            const int rz = cls / (p.str_h * p.str_w), rem = cls - rz * (p.str_h * p.str_w);
+            const int ry = rem / p.str_w, rx = rem - ry * p.str_w;
+            const TapEntry d = mtaps[mt];
+            const int t = rz + p.pad_d - d.dz * p.str_d, rr = ry + p.pad_h - d.dy * p.str_h,
+                      ss = rx + p.pad_w - d.dx * p.str_w;
+            if ((unsigned)t < (unsigned)p.T && (unsigned)rr < (unsigned)p.R && (unsigned)ss < (unsigned)p.S)
+                v = F[((long)c * RST + (t * p.R + rr) * p.S + ss) * p.K + k];
+        }
+        out[e] = v;
+    }
+}
+
+template <typename T, bool BLOCKED, int BM, int BN, int BK, int WM, int WN>
+static int bprop_merged(const ConvPlan& pl, const T* Fm, const void* E, void* gradI, float alpha, hipStream_t stream)
+{
+    const ng_conv_params& p = pl.p;
+    const int ncols = pl.m_nz * pl.m_ny * pl.m_nx * p.N;
+    const int MPQN = p.M * p.P * p.Q * p.N;
+    const int J = pl.m_taps * p.K;
+    const PixelLattice lat = PixelLattice::make(p.N, ncols, pl.m_nx, pl.m_nx * pl.m_ny);
+    DenseLoader<T, MC, true> al{Fm, 0, pl.m_rpad, pl.m_rpad, J};
+    const int nblk = BLOCKED ? p.K / BK : 1;
+    GatherColsLoader<T, T, BLOCKED, BK> bl{(const T*)E, BLOCKED ? pl.d_merged_taps : pl.d_merged_flat, J, lat,
+                                           1, 1, 1, p.M, p.P, p.Q, MPQN, FastDiv::make((unsigned)nblk), nblk};
+    MergedLatticeStoreEpilogue<T> epi{(T*)gradI, pl.m_rows, p.C, FastDiv::make((unsigned)p.C),
+                                      FastDiv::make((unsigned)(p.str_h * p.str_w)), FastDiv::make((unsigned)p.str_w),
+                                      (long)p.D * p.H * p.W * p.N, lat, p.str_d, p.str_h, p.str_w, p.D, p.H, p.W, alpha};
+    return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, epi, pl.m_rows, ncols, cdiv(J, BK), 1, stream,
+                                                      "conv bprop (merged)");
+}
+
+template <typename T, bool BLOCKED>
+static int run_bprop_merged(const ConvPlan& pl, const void* F, const void* E, void* gradI, float alpha, void* ws,
+                            hipStream_t stream)
+{
+    const ng_conv_params& p = pl.p;
+    T* Fm = (T*)ws;
+    const long total = (long)pl.m_taps * p.K * pl.m_rpad;
+    const int blocks = (int)std::min<long>((total + 255) / 256, 4096);
+    hipLaunchKernelGGL(filter_merge_kernel<T>, dim3(blocks), dim3(256), 0, stream, (const T*)F, Fm,
+                       pl.d_merged_taps, p, pl.m_taps, pl.m_rows, pl.m_rpad);
+    NG_CHECK_LAUNCH("filter merge");
+    if constexpr (sizeof(T) == 2) {
+        switch (pick_row_tile(pl.m_rows, pl.m_nz * pl.m_ny * pl.m_nx * p.N, 256)) {
+        case 256: return bprop_merged<T, BLOCKED, 256, 256, 64, 2, 4>(pl, Fm, E, gradI, alpha, stream);
+        case 128: return bprop_merged<T, BLOCKED, 128, 256, 64, 1, 4>(pl, Fm, E, gradI, alpha, stream);
+        default:  return bprop_merged<T, BLOCKED, 64, 256, 64, 1, 4>(pl, Fm, E, gradI, alpha, stream);
+        }
+    } else {
+        return bprop_merged<T, BLOCKED, 128, 128, 16, 2, 2>(pl, Fm, E, gradI, alpha, stream);
     }
 }
 
@@ -68,6 +142,9 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
     const ng_conv_params& p = pl.p;
     if (ws_bytes < pl.ws_bprop || !ws)
         return fail(-40, "ng_conv_bprop: workspace too small (%zu < %zu)", ws_bytes, pl.ws_bprop);
+    if (pl.merged)
+        return (p.K % pl.bk == 0) ? run_bprop_merged<T, true>(pl, F, E, gradI, alpha, ws, stream)
+                                  : run_bprop_merged<T, false>(pl, F, E, gradI, alpha, ws, stream);
     T* Fs = (T*)ws;
     {
         const long total = (long)pl.RST * p.K * pl.Cpad;

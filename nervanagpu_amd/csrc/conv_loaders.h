@@ -325,4 +325,40 @@ struct LatticeStoreEpilogue {
     }
 };
 
+// Epilogue of the merged strided data gradient: row (class, c), column
+// (lattice point, n) lands on input pixel residue(class) + stride * lattice
+// point, if that pixel exists.
+template <typename T>
+struct MergedLatticeStoreEpilogue {
+    typedef typename StoreBits<T>::bits_t bits_t;
+    T*           out;
+    int          rows;         // classes * C
+    int          C;
+    FastDiv      div_c, div_hw, div_w;   // C, str_h*str_w, str_w
+    long         chan_stride;  // D*H*W*N
+    PixelLattice lat;
+    int          sz, sy, sx;
+    int          D, H, W;
+    float        alpha;
+
+    __device__ __forceinline__ void store8(int i, int j0, int /*z*/, int /*split*/, const float (&acc)[8]) const
+    {
+        if (i >= rows || j0 >= lat.ncols) return;
+        const int cls = (int)div_c.div((unsigned)i), c = i - cls * C;
+        const int rz = (int)div_hw.div((unsigned)cls), rem = cls - rz * (sy * sx);
+        const int ry = (int)div_w.div((unsigned)rem), rx = rem - ry * sx;
+        int iz, iy, ix, nn;
+        lat.split(j0, iz, iy, ix, nn);
+        const int z = rz + sz * iz, y = ry + sy * iy, x = rx + sx * ix;
+        if (z >= D || y >= H || x >= W) return;
+        bits_t* p = reinterpret_cast<bits_t*>(out + c * chan_stride + (long)((z * H + y) * W + x) * lat.N + nn);
+        bits_t b[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) b[e] = StoreBits<T>::round(acc[e] * alpha, 0, 0, 0, 0);
+        constexpr int NV = (int)sizeof(bits_t) * 8 / 16;
+#pragma unroll
+        for (int q = 0; q < NV; q++) reinterpret_cast<uint4_t*>(p)[q] = reinterpret_cast<const uint4_t*>(b)[q];
+    }
+};
+
 }  // namespace ng

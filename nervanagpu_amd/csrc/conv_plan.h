@@ -30,6 +30,15 @@ struct ConvPlan {
     TapEntry* d_bprop_taps = nullptr;   // RST entries grouped by class
     int* d_tap_dest = nullptr;          // RST ints: first re-laid filter row of each tap
     std::vector<BpropClass> classes;
+    // Merged form of the strided data gradient (used when all classes together
+    // have at most 256 rows): one problem whose rows are (class, c) and whose
+    // contraction runs over the union of the classes' output-pixel offsets.
+    bool merged = false;
+    int m_rows = 0, m_rpad = 0;         // classes * C and its multiple of 8
+    int m_taps = 0;                     // distinct (dz,dy,dx) offsets
+    int m_nz = 0, m_ny = 0, m_nx = 0;   // lattice of class 0 (the largest)
+    TapEntry* d_merged_taps = nullptr;  // m_taps entries
+    TapEntry* d_merged_flat = nullptr;  // m_taps * K entries, rows (offset, k)
     size_t ws_bprop = 0, ws_update = 0;
 };
 

@@ -83,6 +83,34 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
                 pl->classes.push_back(c);
             }
 
+    // merged strided data gradient: offsets d = (residue + pad - tap) / stride over
+    // all classes span a small box; every (dz,dy,dx) of the box is one merged tap
+    std::vector<TapEntry> mtaps, mflat;
+    const int nclasses = p.str_d * p.str_h * p.str_w;
+    if (nclasses > 1 && (long)nclasses * p.C <= 256) {
+        auto lo = [](int pad, int win, int str) {       // floor((pad - (win-1)) / str)
+            const int a = pad - (win - 1);
+            return a >= 0 ? a / str : -((-a + str - 1) / str);
+        };
+        auto hi = [](int pad, int str) { return (str - 1 + pad) / str; };
+        const int z0 = lo(p.pad_d, p.T, p.str_d), z1 = hi(p.pad_d, p.str_d);
+        const int y0 = lo(p.pad_h, p.R, p.str_h), y1 = hi(p.pad_h, p.str_h);
+        const int x0 = lo(p.pad_w, p.S, p.str_w), x1 = hi(p.pad_w, p.str_w);
+        for (int dz = z0; dz <= z1; dz++)
+            for (int dy = y0; dy <= y1; dy++)
+                for (int dx = x0; dx <= x1; dx++) {
+                    mtaps.push_back(TapEntry{(int)(((long)dz * PQ + dy * p.Q + dx) * p.N), dz, dy, dx});
+                    for (int k = 0; k < p.K; k++)
+                        mflat.push_back(TapEntry{(int)(((long)k * p.M * PQ + (long)dz * PQ + dy * p.Q + dx) * p.N),
+                                                 dz, dy, dx});
+                }
+        pl->merged = true;
+        pl->m_rows = nclasses * p.C;
+        pl->m_rpad = cdiv(pl->m_rows, 8) * 8;
+        pl->m_taps = (int)mtaps.size();
+        pl->m_nz = cdiv(p.D, p.str_d); pl->m_ny = cdiv(p.H, p.str_h); pl->m_nx = cdiv(p.W, p.str_w);
+    }
+
     auto upload = [&](const void* src, size_t bytes, void** dst) -> int {
         if (bytes == 0) { *dst = nullptr; return 0; }
         NG_HIP(hipMalloc(dst, bytes));
@@ -94,9 +122,13 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
     if (!rc) rc = upload(bflat.data(), bflat.size() * sizeof(TapEntry), (void**)&pl->d_bprop_flat);
     if (!rc) rc = upload(btaps.data(), btaps.size() * sizeof(TapEntry), (void**)&pl->d_bprop_taps);
     if (!rc) rc = upload(tap_dest.data(), tap_dest.size() * sizeof(int), (void**)&pl->d_tap_dest);
+    if (!rc) rc = upload(mtaps.data(), mtaps.size() * sizeof(TapEntry), (void**)&pl->d_merged_taps);
+    if (!rc) rc = upload(mflat.data(), mflat.size() * sizeof(TapEntry), (void**)&pl->d_merged_flat);
     if (rc) { ng_conv_plan_destroy(pl); return rc; }
 
     pl->ws_bprop = align_up((size_t)pl->RST * p.K * pl->Cpad * dtype_size(dtype), 256);
+    if (pl->merged)
+        pl->ws_bprop = std::max(pl->ws_bprop, align_up((size_t)pl->m_taps * p.K * pl->m_rpad * dtype_size(dtype), 256));
     {
         const int kt = cdiv(p.M * p.P * p.Q * p.N, pl->bk);
         // the most slices any tile shape of the update dispatcher would ask for
@@ -117,6 +149,8 @@ int ng_conv_plan_destroy(void* plan)
     if (pl->d_bprop_flat) (void)hipFree(pl->d_bprop_flat);
     if (pl->d_bprop_taps) (void)hipFree(pl->d_bprop_taps);
     if (pl->d_tap_dest) (void)hipFree(pl->d_tap_dest);
+    if (pl->d_merged_taps) (void)hipFree(pl->d_merged_taps);
+    if (pl->d_merged_flat) (void)hipFree(pl->d_merged_flat);
     delete pl;
     return 0;
 }

@@ -19,6 +19,7 @@ SMALL = [
     (8, 16, 32, 5, 9, 8, 3, 3, 3, (1, 0, 1), (1, 1, 2)),          # 3-D
     (64, 8, 8, 1, 7, 7, 1, 1, 1, (0, 0, 0), (1, 1, 1)),           # 1x1
     (8, 20, 24, 1, 12, 12, 1, 2, 2, (0, 0, 0), (1, 3, 3)),        # stride > filter: unreached input pixels
+    (8, 72, 64, 1, 12, 11, 1, 3, 3, (0, 1, 1), (1, 2, 2)),        # strided, classes * C > 256: one launch per class
 ]
 
 
