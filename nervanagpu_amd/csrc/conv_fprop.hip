@@ -36,7 +36,13 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
     switch (pick_row_tile(pl.p.K, pl.p.M * pl.p.P * pl.p.Q * pl.p.N, 256)) {
     case 256: return fprop_tile<_Float16, TIN, BLOCKED, 256, 256, 64, 2, 4>(pl, I, F, O, alpha, flags, st);
     case 128: return fprop_tile<_Float16, TIN, BLOCKED, 128, 256, 64, 1, 4>(pl, I, F, O, alpha, flags, st);
-    default:  return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 64, 1, 4>(pl, I, F, O, alpha, flags, st);
+    default:
+        // a first layer's whole contraction (C*T*R*S <= 32) fits a half-depth
+        // tile: half the LDS, twice the workgroups per CU for a kernel that is
+        // all prologue and epilogue
+        if (!BLOCKED && pl.CRST <= 32)
+            return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 32, 1, 4>(pl, I, F, O, alpha, flags, st);
+        return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 64, 1, 4>(pl, I, F, O, alpha, flags, st);
     }
 }
 

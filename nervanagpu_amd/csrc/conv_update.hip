@@ -53,6 +53,8 @@ static int update_h(const ConvPlan& pl, const void* I, const void* E, void* grad
             // and fp32 partials: worth it only for long pixel ranges
             if (pl.p.K >= 256 && pl.CRST >= 256 && (long)pl.p.M * pl.p.P * pl.p.Q * pl.p.N >= 512 * 64)
                 return launch_update<_Float16, TIN, TOUT, true, 256, 256, 64, 2, 4>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
+            if (pl.p.K <= 64 && pl.CRST <= 64)
+                return launch_update<_Float16, TIN, TOUT, true, 64, 64, 64, 2, 2>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
             if (pl.p.K <= 64)
                 return launch_update<_Float16, TIN, TOUT, true, 128, 64, 64, 2, 2>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
         }
