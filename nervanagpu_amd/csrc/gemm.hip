@@ -30,7 +30,8 @@ static int choose_splits(int out_tiles, int total_k_tiles, size_t slice_bytes, s
 {
     const int cus = device_cu_count();
     if (out_tiles >= cus || total_k_tiles < 8) return 1;
-    int splits = ceil_div(2 * cus, out_tiles);
+    // about one and a half workgroups per CU: more slices only add fp32 partials
+    int splits = ceil_div(3 * cus / 2, out_tiles);
     splits = std::min(splits, total_k_tiles / 4);
     if (slice_bytes) splits = (int)std::min<size_t>((size_t)splits, ws_bytes / slice_bytes);
     // every slice must own at least one tile

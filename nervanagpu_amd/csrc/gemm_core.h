@@ -276,6 +276,15 @@ struct InterleaveStep {
 // staging -> 8-column chunks handed to the epilogue functor.  The band index is
 // a template parameter so that every accumulator access is a static register
 // reference.
+// The staging region of the epilogue is private to a wavefront and LDS
+// operations of one wavefront execute in order, so write -> read -> rewrite only
+// needs the compiler kept from reordering them; no workgroup barrier.
+__device__ __forceinline__ void wave_lds_fence()
+{
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
 template <int TM, int TN, int WTN, int EPITCH, int I>
 struct EpilogueBands {
     template <class Epi>
@@ -291,7 +300,7 @@ struct EpilogueBands {
             for (int v = 0; v < 16; v++)
                 *reinterpret_cast<float*>(stage + ((v >> 2) * 8 + rsub + (v & 3)) * EPITCH + (j * 32 + col) * 4) =
                     acc[I][j][v];
-        __syncthreads();
+        wave_lds_fence();
 #pragma unroll
         for (int c = 0; c < CPW / 64; c++) {
             const int id = lane + c * 64;
@@ -302,7 +311,7 @@ struct EpilogueBands {
             const float vals[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             epi.store8(mbase + I * 32 + r, nbase + cc, z, split, vals);
         }
-        __syncthreads();
+        wave_lds_fence();
         if constexpr (I + 1 < TM)
             EpilogueBands<TM, TN, WTN, EPITCH, I + 1>::run(acc, stage, lane, mbase, nbase, z, split, epi);
     }
