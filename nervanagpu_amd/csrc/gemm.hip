@@ -117,7 +117,12 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
     // minibatch-wide outputs (n <= 128) stream the weight matrix: halve the row
     // tile so that fewer contraction slices, i.e. fewer fp32 partials, fill the chip
     const long tiles128 = (long)ceil_div(g.m, 128) * ceil_div(g.n, 128) * g.batch_grid;
-    if (tiles128 >= cus) return launch_layout<_Float16, 128, 128, 64, 2, 2, true>(g, sr_bits);
+    if (tiles128 >= cus) {
+        // short contractions are all prologue and epilogue: half-depth tiles halve
+        // the LDS footprint, so more workgroups overlap their loads and stores
+        if (k_tiles <= 4) return launch_layout<_Float16, 128, 128, 32, 2, 2, true>(g, sr_bits);
+        return launch_layout<_Float16, 128, 128, 64, 2, 2, true>(g, sr_bits);
+    }
     if (g.n <= 128) return launch_layout<_Float16, 64, 128, 64, 2, 2, true>(g, sr_bits);
     // mid-sized outputs: small tiles fill the chip without (or with fewer)
     // contraction slices, which cost fp32 partials and a second launch
