@@ -776,10 +776,48 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
         __builtin_amdgcn_s_waitcnt(WaitVmLgkm0<(NSTAGE - 2) * N_CHUNKS>::IMM);
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
-        gissue(rd_off);
-        __builtin_amdgcn_sched_barrier(0);
-        rd_off = next_stage(rd_off);
-        step(rd_off, 0, fa[NSTEP & 1], fb[NSTEP & 1], fa[(NSTEP - 1) & 1], fb[(NSTEP - 1) & 1]);
+        if constexpr (N_MFMA >= 8) {
+            // Last k-step of tile t with the requests for tile t+NSTAGE and the
+            // first fragment reads of tile t+1 placed between its MFMAs by hand,
+            // one request per MFMA: the matrix pipe keeps running behind the
+            // barrier instead of waiting out a burst of requests.  (With fewer
+            // MFMAs per step the requests would outnumber them; those shapes
+            // issue the burst first.)
+            const int wr_off = rd_off;
+            rd_off = next_stage(rd_off);
+            if (!PREP_AHEAD) gprep();
+            const char* tile = smem + rd_off;
+            Frag<T> (&na)[TM] = fa[NSTEP & 1];
+            Frag<T> (&nb)[TN] = fb[NSTEP & 1];
+            const Frag<T> (&ca)[TM] = fa[(NSTEP - 1) & 1];
+            const Frag<T> (&cb)[TN] = fb[(NSTEP - 1) & 1];
+            constexpr int PER = (N_CHUNKS + N_MFMA - 1) / N_MFMA;
+#pragma unroll
+            for (int m = 0; m < N_MFMA; m++) {
+                mfma_step(ca[m / TN], cb[m % TN], acc[m / TN][m % TN]);
+                if (m < TM) na[m < TM ? m : 0] = FA::load(tile, fa_base[m < TM ? m : 0], 0);
+                else if (m < TM + TN) nb[m - TM < TN ? (m >= TM ? m - TM : 0) : 0] = FB::load(tile, fb_base[m - TM < TN ? (m >= TM ? m - TM : 0) : 0], 0);
+#pragma unroll
+                for (int q = 0; q < PER; q++) {
+                    const int c = m * PER + q;
+                    if (c < CPT_A) {
+                        const int i = c < CPT_A ? c : 0;
+                        buffer_load_chunk_to_lds(g_ta.rsrc, smem + wr_off + (i * NT + wave * 64) * 16, aload.offset(g_ta, actx[i]));
+                    } else if (c < N_CHUNKS) {
+                        const int i = (c >= CPT_A && c < N_CHUNKS) ? c - CPT_A : 0;
+                        buffer_load_chunk_to_lds(g_tb.rsrc, smem + wr_off + TA::BYTES + (i * NT + wave * 64) * 16,
+                                                 bload.offset(g_tb, bctx[i]));
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (PREP_AHEAD) gprep();
+        } else {
+            gissue(rd_off);
+            __builtin_amdgcn_sched_barrier(0);
+            rd_off = next_stage(rd_off);
+            step(rd_off, 0, fa[NSTEP & 1], fb[NSTEP & 1], fa[(NSTEP - 1) & 1], fb[(NSTEP - 1) & 1]);
+        }
     }
     // drain: nothing left to request
     for (; t + 1 < ntiles; t++) {
