@@ -27,6 +27,21 @@ template <> struct Pack<float, 4>    { typedef uint4 raw_t; };
 template <> struct Pack<_Float16, 1> { typedef unsigned short raw_t; };
 template <> struct Pack<float, 1>    { typedef unsigned raw_t; };
 
+// non-temporal load of a 2-, 4- or 16-byte packet
+template <typename R>
+__device__ __forceinline__ R load_streaming(const R* p)
+{
+    if constexpr (sizeof(R) == 16) {
+        typedef unsigned v4u __attribute__((ext_vector_type(4)));
+        const v4u v = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(p));
+        return __builtin_bit_cast(R, v);
+    } else if constexpr (sizeof(R) == 4) {
+        return __builtin_bit_cast(R, __builtin_nontemporal_load(reinterpret_cast<const unsigned*>(p)));
+    } else {
+        return __builtin_bit_cast(R, __builtin_nontemporal_load(reinterpret_cast<const unsigned short*>(p)));
+    }
+}
+
 template <typename T, int VEC>
 __device__ __forceinline__ void load_vec(const T* p, float (&v)[VEC])
 {
@@ -60,6 +75,9 @@ struct PoolGeom {
     // (fprop kernels: Q, P; bprop gather: W, H); window ranges divide by strides
     FastDiv div_nvec, div_q, div_p, div_w, div_h;
     FastDiv div_sj, div_sd, div_sh, div_sw;
+    // input read exactly once (windows do not overlap) and larger than the
+    // last-level cache: streamed with non-temporal loads
+    int stream_in;
 };
 
 enum { OP_MAX = 0, OP_AVG = 1 };
@@ -118,7 +136,8 @@ void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char
             const int y = y0 + tap / (RS > 0 ? RS : 1), x = x0 + tap % (RS > 0 ? RS : 1);
             ok[tap] = plane_ok && (unsigned)y < (unsigned)g.H && (unsigned)x < (unsigned)g.W;
             const T* src = ok[tap] ? plane + ((long)y * g.W + x) * g.N : Inv;
-            raw[tap] = *reinterpret_cast<const raw_t*>(src);
+            raw[tap] = g.stream_in ? load_streaming(reinterpret_cast<const raw_t*>(src))
+                                   : *reinterpret_cast<const raw_t*>(src);
         }
 #pragma unroll
         for (int tap = 0; tap < NTAP; tap++) {
@@ -303,7 +322,7 @@ void pool_bprop_kernel(const T* __restrict__ E, const unsigned char* __restrict_
 // windows that tile the input exactly (stride == window, no padding, extents
 // divisible): one thread owns a whole window and writes all of its grad_I
 // elements, so max bprop needs a single pass and no argmax scratch.
-template <typename T, int VEC>
+template <typename T, int VEC, int RS>
 __global__ __launch_bounds__(256)
 void pool_bprop_max_tiled_kernel(const T* __restrict__ I, const T* __restrict__ E, T* __restrict__ B, PoolGeom g)
 {
@@ -316,6 +335,40 @@ void pool_bprop_max_tiled_kernel(const T* __restrict__ I, const T* __restrict__ 
     const long in_base = ((((long)c0 * g.D + z0) * g.H + y0) * g.W + x0) * g.N + (long)nv * VEC;
     const long sx = g.N, sy = (long)g.W * g.N, sz = (long)g.H * g.W * g.N, sc = (long)g.D * g.H * g.W * g.N;
 
+    if (RS > 0) {
+        // 2-D RS x RS window known at compile time: all loads, then all stores
+        constexpr int NTAP = RS > 0 ? RS * RS : 1;
+        typedef typename Pack<T, VEC>::raw_t raw_t;
+        raw_t raw[NTAP];
+#pragma unroll
+        for (int tap = 0; tap < NTAP; tap++) {
+            const raw_t* src = reinterpret_cast<const raw_t*>(I + in_base + (tap / (RS > 0 ? RS : 1)) * sy + (tap % (RS > 0 ? RS : 1)) * sx);
+            raw[tap] = g.stream_in ? load_streaming(src) : *src;
+        }
+        float ev[VEC];
+        load_vec<T, VEC>(E + ((long)k * per_map + inner) * VEC, ev);
+        float best[VEC];
+        int   slot_of[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; i++) { best[i] = -NG_FLT_MAX; slot_of[i] = 0; }
+#pragma unroll
+        for (int tap = 0; tap < NTAP; tap++) {
+            const T* e = reinterpret_cast<const T*>(&raw[tap]);
+#pragma unroll
+            for (int i = 0; i < VEC; i++) {
+                const float v = (float)e[i];
+                if (v > best[i]) { best[i] = v; slot_of[i] = tap; }
+            }
+        }
+#pragma unroll
+        for (int tap = 0; tap < NTAP; tap++) {
+            float out[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; i++) out[i] = (slot_of[i] == tap) ? ev[i] : 0.0f;
+            store_vec<T, VEC>(B + in_base + (tap / (RS > 0 ? RS : 1)) * sy + (tap % (RS > 0 ? RS : 1)) * sx, out);
+        }
+        return;
+    }
     float best[VEC];
     int   slot_of[VEC];
 #pragma unroll
@@ -345,7 +398,7 @@ void pool_bprop_max_tiled_kernel(const T* __restrict__ I, const T* __restrict__ 
                 }
 }
 
-static PoolGeom make_geom(const ng_pool_params& p, int vec)
+static PoolGeom make_geom(const ng_pool_params& p, int vec, size_t elem_bytes)
 {
     PoolGeom g{p.N, p.C, p.D, p.H, p.W, p.J, p.T, p.R, p.S, p.K, p.M, p.P, p.Q,
                p.pad_j, p.pad_d, p.pad_h, p.pad_w, p.str_j, p.str_d, p.str_h, p.str_w, p.N / vec};
@@ -358,6 +411,9 @@ static PoolGeom make_geom(const ng_pool_params& p, int vec)
     g.div_sd = FastDiv::make((unsigned)p.str_d);
     g.div_sh = FastDiv::make((unsigned)p.str_h);
     g.div_sw = FastDiv::make((unsigned)p.str_w);
+    const bool disjoint = p.str_j >= p.J && p.str_d >= p.T && p.str_h >= p.R && p.str_w >= p.S;
+    const size_t in_bytes = (size_t)p.C * p.D * p.H * p.W * p.N * elem_bytes;
+    g.stream_in = (disjoint && in_bytes > (256u << 20)) ? 1 : 0;
     return g;
 }
 
@@ -406,7 +462,7 @@ static void launch_fprop(const PoolGeom& g, int rs, dim3 grid, const T* I, T* O,
 template <typename T, int VEC>
 static int run_fprop(const ng_pool_params& p, int op, const void* I, void* O, hipStream_t st)
 {
-    PoolGeom g = make_geom(p, VEC);
+    PoolGeom g = make_geom(p, VEC, sizeof(T));
     const dim3 grid = grid_for((long)g.M * g.P * g.Q * g.nvec, g.K);
     const int rs = square_window(p);
     if (op == OP_MAX) launch_fprop<T, VEC, OP_MAX, false>(g, rs, grid, (const T*)I, (T*)O, nullptr, st);
@@ -435,7 +491,7 @@ template <typename T, int VEC>
 static int run_bprop(const ng_pool_params& p, int op, const void* I, const void* E, void* B,
                      void* ws, size_t ws_bytes, hipStream_t st)
 {
-    PoolGeom g = make_geom(p, VEC);
+    PoolGeom g = make_geom(p, VEC, sizeof(T));
     const long out_total = (long)g.K * g.M * g.P * g.Q * g.nvec;
     const dim3 out_grid = grid_for((long)g.M * g.P * g.Q * g.nvec, g.K);
     const dim3 in_grid = grid_for((long)g.D * g.H * g.W * g.nvec, g.C);
@@ -446,8 +502,16 @@ static int run_bprop(const ng_pool_params& p, int op, const void* I, const void*
         return 0;
     }
     if (tiles_exactly(p)) {
-        hipLaunchKernelGGL((pool_bprop_max_tiled_kernel<T, VEC>), out_grid, dim3(256), 0, st,
-                           (const T*)I, (const T*)E, (T*)B, g);
+        const int rs = (VEC > 1) ? square_window(p) : 0;
+        if (rs == 2)
+            hipLaunchKernelGGL((pool_bprop_max_tiled_kernel<T, VEC, 2>), out_grid, dim3(256), 0, st,
+                               (const T*)I, (const T*)E, (T*)B, g);
+        else if (rs == 3)
+            hipLaunchKernelGGL((pool_bprop_max_tiled_kernel<T, VEC, 3>), out_grid, dim3(256), 0, st,
+                               (const T*)I, (const T*)E, (T*)B, g);
+        else
+            hipLaunchKernelGGL((pool_bprop_max_tiled_kernel<T, VEC, 0>), out_grid, dim3(256), 0, st,
+                               (const T*)I, (const T*)E, (T*)B, g);
         NG_CHECK_LAUNCH("pool max bprop (tiled)");
         return 0;
     }
