@@ -78,6 +78,9 @@ struct PoolGeom {
     // input read exactly once (windows do not overlap) and larger than the
     // last-level cache: streamed with non-temporal loads
     int stream_in;
+    // forward kernels with overlapping windows and many workgroups per feature
+    // map: XCD-contiguous workgroup numbering (gridDim.x padded to a multiple of 8)
+    int xcd_remap;
 };
 
 enum { OP_MAX = 0, OP_AVG = 1 };
@@ -87,6 +90,15 @@ enum { OP_MAX = 0, OP_AVG = 1 };
 // Launch geometry shared by the kernels: blockIdx.y is the outermost index
 // (output or input feature map), blockIdx.x * 256 + threadIdx.x the position
 // inside that map: ((d * H + h) * W + w) * nvec + nv, below 2^31.
+// Workgroups are dealt to the 8 XCDs round robin by linear id.  With gridDim.x a
+// multiple of 8, the XCD of a workgroup is blockIdx.x % 8; renumbering gives
+// each XCD one contiguous eighth of every feature map, and rows shared by
+// overlapping windows are fetched into one L2 instead of several.
+__device__ __forceinline__ unsigned xcd_block_index(int remap)
+{
+    return remap ? (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3) : blockIdx.x;
+}
+
 __device__ __forceinline__ bool split_inner(unsigned inner, unsigned limit, const FastDiv& dn, const FastDiv& d1,
                                             const FastDiv& d2, int nvec, int e1, int e2, int& nv, int& i1, int& i2,
                                             int& i3)
@@ -111,7 +123,7 @@ __global__ __launch_bounds__(256)
 void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char* __restrict__ arg, PoolGeom g)
 {
     const unsigned per_map = (unsigned)(g.M * g.P * g.Q * g.nvec);
-    const unsigned inner = blockIdx.x * 256u + threadIdx.x;
+    const unsigned inner = xcd_block_index(g.xcd_remap) * 256u + threadIdx.x;
     const int k = blockIdx.y;
     int nv, q, p, m;
     if (!split_inner(inner, per_map, g.div_nvec, g.div_q, g.div_p, g.nvec, g.Q, g.P, nv, q, p, m)) return;
@@ -414,6 +426,7 @@ static PoolGeom make_geom(const ng_pool_params& p, int vec, size_t elem_bytes)
     const bool disjoint = p.str_j >= p.J && p.str_d >= p.T && p.str_h >= p.R && p.str_w >= p.S;
     const size_t in_bytes = (size_t)p.C * p.D * p.H * p.W * p.N * elem_bytes;
     g.stream_in = (disjoint && in_bytes > (256u << 20)) ? 1 : 0;
+    g.xcd_remap = (!disjoint && (long)p.M * p.P * p.Q * g.nvec >= 16 * 256) ? 1 : 0;
     return g;
 }
 
@@ -439,7 +452,12 @@ static int check_params(const ng_pool_params& p, int dtype, int op)
 }
 
 // grid over (positions of one feature map) x (feature maps)
-static dim3 grid_for(long per_map, int maps) { return dim3((unsigned)((per_map + 255) / 256), (unsigned)maps, 1); }
+static dim3 grid_for(long per_map, int maps, int pad8 = 0)
+{
+    unsigned blocks = (unsigned)((per_map + 255) / 256);
+    if (pad8) blocks = (blocks + 7u) / 8u * 8u;   // see xcd_block_index()
+    return dim3(blocks, (unsigned)maps, 1);
+}
 
 // compile-time window size of the unrolled forward kernels (0: generic loops)
 static int square_window(const ng_pool_params& p)
@@ -463,7 +481,7 @@ template <typename T, int VEC>
 static int run_fprop(const ng_pool_params& p, int op, const void* I, void* O, hipStream_t st)
 {
     PoolGeom g = make_geom(p, VEC, sizeof(T));
-    const dim3 grid = grid_for((long)g.M * g.P * g.Q * g.nvec, g.K);
+    const dim3 grid = grid_for((long)g.M * g.P * g.Q * g.nvec, g.K, g.xcd_remap);
     const int rs = square_window(p);
     if (op == OP_MAX) launch_fprop<T, VEC, OP_MAX, false>(g, rs, grid, (const T*)I, (T*)O, nullptr, st);
     else              launch_fprop<T, VEC, OP_AVG, false>(g, rs, grid, (const T*)I, (T*)O, nullptr, st);
@@ -493,7 +511,7 @@ static int run_bprop(const ng_pool_params& p, int op, const void* I, const void*
 {
     PoolGeom g = make_geom(p, VEC, sizeof(T));
     const long out_total = (long)g.K * g.M * g.P * g.Q * g.nvec;
-    const dim3 out_grid = grid_for((long)g.M * g.P * g.Q * g.nvec, g.K);
+    const dim3 out_grid = grid_for((long)g.M * g.P * g.Q * g.nvec, g.K, g.xcd_remap);
     const dim3 in_grid = grid_for((long)g.D * g.H * g.W * g.nvec, g.C);
     const bool win2 = two_window_cover(p);
     if (op == OP_AVG) {
