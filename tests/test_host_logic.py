@@ -201,3 +201,13 @@ def test_magic32(nmax, d):
     n = np.arange(nmax + 1, dtype=np.uint64)
     assert np.array_equal(n // d, (n * m) >> s)
     assert L._flatten([1, [2, (3, [4])], 5]) == [1, 2, 3, 4, 5]
+
+
+def test_network_tables_and_flops():
+    """host logic only: the four benchmark networks chain their geometry like the
+    reference tables (benchmarks/convnet-benchmarks.py:120-200)"""
+    from nervanagpu_amd import convnet_benchmarks as cb
+    assert len(cb.network_config("Alexnet")) == 12
+    assert len(cb.network_config("VGG")) == 17
+    assert len(cb.network_config("VGG_E")) == 25
+    assert cb.PUBLISHED_TITAN_X_MS[("VGG", "float16")][2] == 491.382
