@@ -23,9 +23,11 @@ import sys
 import numpy as np
 
 from . import NervanaGPU, _lib
-from .layers import Layer, DataLayer, ConvLayer, PoolLayer, FullLayer
+from .layers import Layer, DataLayer, ConvLayer, PoolLayer, FullLayer, Inception
 
-# layer shorthands: ("conv", K, R, pad, stride) / ("pool", R, stride) / ("full", nOut)
+# layer shorthands: ("conv", K, R, pad, stride) / ("pool", R, stride[, pad[, op]]) / ("full", nOut)
+# ("incep1", widths) / ("incep2", widths): the two inception module shapes, see _inception()
+_STEM = [("conv", 64, 7, 3, 2), ("pool", 3, 2, 1), ("conv", 64, 1, 0, 1), ("conv", 192, 3, 1, 1), ("pool", 3, 2, 1)]
 _NETS = {
     "Alexnet": dict(N=128, H=224, warmup=5, layers=[
         ("conv", 64, 11, 2, 4), ("pool", 3, 2), ("conv", 192, 5, 2, 1), ("pool", 3, 2),
@@ -48,6 +50,31 @@ _NETS = {
         [("conv", 512, 3, 1, 1)] * 4 + [("pool", 2, 2)] +
         [("conv", 512, 3, 1, 1)] * 4 + [("pool", 2, 2)] +
         [("full", 3072), ("full", 3072), ("full", 1000)]),
+    # http://arxiv.org/abs/1409.4842
+    "GoogLeNet1": dict(N=128, H=224, warmup=1, layers=_STEM + [
+        ("incep1", ((64,), (96, 128), (16, 32), (32,))),
+        ("incep1", ((128,), (128, 192), (32, 96), (64,))), ("pool", 3, 2, 1),
+        ("incep1", ((192,), (96, 208), (16, 48), (64,))),
+        ("incep1", ((160,), (112, 224), (24, 64), (64,))),
+        ("incep1", ((128,), (128, 256), (24, 64), (64,))),
+        ("incep1", ((112,), (144, 288), (32, 64), (64,))),
+        ("incep1", ((256,), (160, 320), (32, 128), (128,))), ("pool", 3, 2, 1),
+        ("incep1", ((256,), (160, 320), (32, 128), (128,))),
+        ("incep1", ((384,), (192, 384), (48, 128), (128,))),
+        ("pool", 7, 1, 0, "avg"), ("full", 1000)]),
+    # the batch-normalised variant's shapes (http://arxiv.org/abs/1502.03167), without the normalisation
+    "GoogLeNet2": dict(N=128, H=224, warmup=1, layers=_STEM + [
+        ("incep2", ((64,), (64, 64), (64, 96), ("avg", 32))),
+        ("incep2", ((64,), (64, 96), (64, 96), ("avg", 64))),
+        ("incep2", ((0,), (128, 160), (64, 96), ("max", 0))), ("conv", 576, 2, 0, 2),
+        ("incep2", ((224,), (64, 96), (96, 128), ("avg", 128))),
+        ("incep2", ((192,), (96, 128), (96, 128), ("avg", 128))),
+        ("incep2", ((160,), (128, 160), (128, 160), ("avg", 96))),
+        ("incep2", ((96,), (128, 192), (160, 192), ("avg", 96))),
+        ("incep2", ((0,), (128, 192), (192, 256), ("max", 0))), ("conv", 1024, 2, 0, 2),
+        ("incep2", ((352,), (192, 320), (160, 224), ("avg", 128))),
+        ("incep2", ((352,), (192, 320), (192, 224), ("max", 128))),
+        ("pool", 7, 1, 0, "avg"), ("full", 1000)]),
 }
 
 # reference README.md:140-187: (fprop ms, bprop ms, total ms) on one GTX Titan X
@@ -59,18 +86,45 @@ PUBLISHED_TITAN_X_MS = {
 }
 
 
+def _conv(K, R, pad=0, strd=1):
+    return {"layer": ConvLayer, "K": K, "R": R, "S": R, "pad_h": pad, "pad_w": pad, "str_h": strd, "str_w": strd}
+
+
+def _pool(R, strd, pad=0, op="max"):
+    return {"layer": PoolLayer, "op": op, "R": R, "S": R, "str_h": strd, "str_w": strd, "pad_h": pad, "pad_w": pad}
+
+
+def _inception(kind, w):
+    """Inception configuration from its branch widths (reference
+    benchmarks/convnet-benchmarks.py:76-118).  "incep1": 1x1 | 1x1 -> 3x3 |
+    1x1 -> 5x5 | 3x3 max pool -> 1x1.  "incep2": [1x1] | 1x1 -> 3x3 |
+    1x1 -> 3x3 -> 3x3 | 3x3 pool (w[3][0] names the op) [-> 1x1]; a zero width
+    drops the bracketed layer."""
+    if kind == "incep1":
+        parts = [(_conv(w[0][0], 1),),
+                 (_conv(w[1][0], 1), _conv(w[1][1], 3, 1)),
+                 (_conv(w[2][0], 1), _conv(w[2][1], 5, 2)),
+                 (_pool(3, 1, 1), _conv(w[3][0], 1))]
+    else:
+        parts = [(_conv(w[0][0], 1),)] if w[0][0] else []
+        parts += [(_conv(w[1][0], 1), _conv(w[1][1], 3, 1)),
+                  (_conv(w[2][0], 1), _conv(w[2][1], 3, 1), _conv(w[2][1], 3, 1))]
+        tail = (_pool(3, 1, 1, w[3][0]),)
+        parts.append(tail + (_conv(w[3][1], 1),) if w[3][1] else tail)
+    return {"layer": Inception, "partitions": tuple(parts)}
+
+
 def network_config(name):
     """list of Layer.create configuration dicts for a named network"""
     net = _NETS[name]
     confs = [{"layer": DataLayer, "N": net["N"], "C": 3, "H": net["H"], "W": net["H"]}]
     for spec in net["layers"]:
         if spec[0] == "conv":
-            _, K, R, pad, strd = spec
-            confs.append({"layer": ConvLayer, "K": K, "R": R, "S": R, "pad_h": pad, "pad_w": pad,
-                          "str_h": strd, "str_w": strd})
+            confs.append(_conv(*spec[1:]))
         elif spec[0] == "pool":
-            _, R, strd = spec
-            confs.append({"layer": PoolLayer, "op": "max", "R": R, "S": R, "str_h": strd, "str_w": strd})
+            confs.append(_pool(*spec[1:]))
+        elif spec[0] in ("incep1", "incep2"):
+            confs.append(_inception(*spec))
         else:
             confs.append({"layer": FullLayer, "nOut": spec[1]})
     return confs
@@ -91,8 +145,10 @@ def build_network(ng, confs, dtype, zeros=False, seed=0):
         prev = layer
         layers.append(layer)
 
-    # two alternating buffers: a layer cannot read and write its errors in one buffer
-    shared_deltas = [ng.empty(max_delta_layer.dimI, dtype=max_delta_layer.dtype) for _ in range(2)]
+    # two alternating buffers: a layer cannot read and write its errors in one buffer;
+    # the branches inside an inception layer alternate between two more
+    nbuf = 4 if any(type(l) is Inception for l in layers) else 2
+    shared_deltas = [ng.empty(max_delta_layer.dimI, dtype=max_delta_layer.dtype) for _ in range(nbuf)]
     shared_updates = ng.empty(max_weight_layer.dimF, dtype=np.float32)
     np.random.seed(seed)
     for i, layer in enumerate(layers):

@@ -207,7 +207,32 @@ def test_network_tables_and_flops():
     """host logic only: the four benchmark networks chain their geometry like the
     reference tables (benchmarks/convnet-benchmarks.py:120-200)"""
     from nervanagpu_amd import convnet_benchmarks as cb
+    from nervanagpu_amd.layers import Inception
     assert len(cb.network_config("Alexnet")) == 12
     assert len(cb.network_config("VGG")) == 17
     assert len(cb.network_config("VGG_E")) == 25
     assert cb.PUBLISHED_TITAN_X_MS[("VGG", "float16")][2] == 491.382
+
+    # inception modules: output channels are the sum of the branch tails
+    def tail_k(conf):
+        return [part[-1].get("K") for part in conf["partitions"]]
+    g1 = cb.network_config("GoogLeNet1")
+    assert len(g1) == 19 and sum(c["layer"] is Inception for c in g1) == 9
+    assert sum(tail_k(g1[6])) == 256 and sum(tail_k(g1[7])) == 480 and sum(tail_k(g1[-3])) == 1024
+    assert g1[-2]["op"] == "avg" and g1[-2]["R"] == 7 and g1[1]["str_h"] == 2 and g1[1]["pad_h"] == 3
+    g2 = cb.network_config("GoogLeNet2")
+    assert len(g2) == 20 and sum(c["layer"] is Inception for c in g2) == 10
+    assert tail_k(g2[6]) == [64, 64, 96, 32] and [len(p) for p in g2[6]["partitions"]] == [1, 2, 3, 2]
+    # a zero width drops the 1x1 branch and the 1x1 after the pool: the pool passes its channels through
+    assert tail_k(g2[8]) == [160, 96, None] and g2[8]["partitions"][-1][0]["op"] == "max"
+    assert g2[9]["K"] == 576 and g2[9]["R"] == 2 and g2[9]["str_w"] == 2
+
+    # chained through Layer.create: the published GoogLeNet channel / map sizes
+    # (http://arxiv.org/abs/1409.4842 table 1)
+    ng, prev, widths = NervanaGPU(), None, []
+    for conf in g1:
+        prev = L.Layer.create(ng, conf, prev, np.float16)
+        if type(prev) is Inception:
+            widths.append((prev.K, prev.P))
+    assert widths == [(256, 28), (480, 28), (512, 14), (512, 14), (512, 14), (528, 14), (832, 14), (832, 7), (1024, 7)]
+    assert prev.nIn == 1024 and prev.nOut == 1000
