@@ -42,11 +42,22 @@ __device__ __forceinline__ R load_streaming(const R* p)
     }
 }
 
+// One 16-byte (or scalar) load.  The empty asm pins the four words in
+// registers: without it the optimiser may follow the element-wise uses back to
+// the load and split it into 2- and 4-byte pieces of lower alignment.
+template <typename R>
+__device__ __forceinline__ R load_packet(const R* p)
+{
+    R v = *p;
+    if constexpr (sizeof(R) == 16) asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w));
+    return v;
+}
+
 template <typename T, int VEC>
 __device__ __forceinline__ void load_vec(const T* p, float (&v)[VEC])
 {
     typedef typename Pack<T, VEC>::raw_t raw_t;
-    raw_t raw = *reinterpret_cast<const raw_t*>(p);
+    raw_t raw = load_packet(reinterpret_cast<const raw_t*>(p));
     const T* e = reinterpret_cast<const T*>(&raw);
 #pragma unroll
     for (int i = 0; i < VEC; i++) v[i] = (float)e[i];
@@ -81,6 +92,11 @@ struct PoolGeom {
     // forward kernels with overlapping windows and many workgroups per feature
     // map: XCD-contiguous workgroup numbering (gridDim.x padded to a multiple of 8)
     int xcd_remap;
+    // backward by cells (pool_bprop_cell_kernel): which compiled (window, stride)
+    // shape applies (0: none) and the number of stride-sized cells along h and w
+    // that hold at least one input element
+    int use_cells, cells_h, cells_w;
+    FastDiv div_ch, div_cw;
 };
 
 enum { OP_MAX = 0, OP_AVG = 1 };
@@ -112,6 +128,35 @@ __device__ __forceinline__ bool split_inner(unsigned inner, unsigned limit, cons
     i2 = (int)(r1 - r2 * (unsigned)e2);
     i3 = (int)r2;
     return true;
+}
+
+// VEC elements of T as one register vector
+template <typename T, int VEC> struct Lanes {
+    typedef T type __attribute__((ext_vector_type(VEC)));
+    static __device__ __forceinline__ type splat(T v) { return (type)(v); }
+    static __device__ __forceinline__ type max(type a, type b) { return __builtin_elementwise_max(a, b); }
+    static __device__ __forceinline__ T get(const type& a, int i) { return a[i]; }
+};
+template <typename T> struct Lanes<T, 1> {
+    typedef T type;
+    static __device__ __forceinline__ type splat(T v) { return v; }
+    static __device__ __forceinline__ type max(type a, type b) { return a < b ? b : a; }
+    static __device__ __forceinline__ T get(const type& a, int) { return a; }
+};
+
+// argmax slots of VEC elements, one byte each
+template <int VEC>
+__device__ __forceinline__ void store_slots(unsigned char* dst, const int (&slot_of)[VEC])
+{
+    if constexpr (VEC == 8) {
+        uint2 packed;
+        packed.x = (unsigned)slot_of[0] | ((unsigned)slot_of[1] << 8) | ((unsigned)slot_of[2] << 16) | ((unsigned)slot_of[3] << 24);
+        packed.y = (unsigned)slot_of[4] | ((unsigned)slot_of[5] << 8) | ((unsigned)slot_of[6] << 16) | ((unsigned)slot_of[7] << 24);
+        *reinterpret_cast<uint2*>(dst) = packed;
+    } else {
+#pragma unroll
+        for (int i = 0; i < VEC; i++) dst[i] = (unsigned char)slot_of[i];
+    }
 }
 
 // one thread: VEC images of one output element.  RS > 0: the window is a 2-D
@@ -151,17 +196,47 @@ void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char
             raw[tap] = g.stream_in ? load_streaming(reinterpret_cast<const raw_t*>(src))
                                    : *reinterpret_cast<const raw_t*>(src);
         }
+        if constexpr (OP == OP_MAX) {
+            // Branch-free, in the element type: the running maximum over all taps
+            // (two fp16 elements per instruction), then a scan from the last tap
+            // to the first for the first one that holds it: the element the
+            // reference's strict '>' scan keeps.  Taps outside the image become -inf.
+            typedef typename Lanes<T, VEC>::type lanes_t;
+            const T lowest = (T)(-__builtin_huge_valf());
+            lanes_t taps[NTAP];
+            bool all_ok = true;
 #pragma unroll
-        for (int tap = 0; tap < NTAP; tap++) {
-            const T* e = reinterpret_cast<const T*>(&raw[tap]);
+            for (int tap = 0; tap < NTAP; tap++) {
+                taps[tap] = __builtin_bit_cast(lanes_t, raw[tap]);
+                all_ok = all_ok && ok[tap];
+            }
+            if (!all_ok) {
 #pragma unroll
-            for (int i = 0; i < VEC; i++) {
-                const float v = (float)e[i];
-                if (OP == OP_MAX) {
-                    if (ok[tap] && v > best[i]) { best[i] = v; slot_of[i] = tap; }
-                } else {
-                    best[i] += ok[tap] ? v : 0.0f;
+                for (int tap = 0; tap < NTAP; tap++)
+                    if (!ok[tap]) taps[tap] = Lanes<T, VEC>::splat(lowest);
+            }
+            lanes_t top = taps[0];
+#pragma unroll
+            for (int tap = 1; tap < NTAP; tap++) top = Lanes<T, VEC>::max(top, taps[tap]);
+            const long o = ((long)k * per_map + inner) * VEC;
+            if constexpr (!WRITE_ARG) {
+                *reinterpret_cast<raw_t*>(O + o) = __builtin_bit_cast(raw_t, top);
+            } else {
+#pragma unroll
+                for (int tap = NTAP - 1; tap >= 0; tap--) {
+#pragma unroll
+                    for (int i = 0; i < VEC; i++)
+                        slot_of[i] = (Lanes<T, VEC>::get(taps[tap], i) == Lanes<T, VEC>::get(top, i)) ? tap : slot_of[i];
                 }
+                store_slots<VEC>(arg + o, slot_of);
+            }
+            return;
+        } else {
+#pragma unroll
+            for (int tap = 0; tap < NTAP; tap++) {
+                const T* e = reinterpret_cast<const T*>(&raw[tap]);
+#pragma unroll
+                for (int i = 0; i < VEC; i++) best[i] += ok[tap] ? (float)e[i] : 0.0f;
             }
         }
     } else {
@@ -197,16 +272,7 @@ void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char
     }
     const long o = ((long)k * per_map + inner) * VEC;
     if (WRITE_ARG) {
-        if (VEC == 8) {
-            uint2 packed;
-            packed.x = (unsigned)slot_of[0] | ((unsigned)slot_of[1] << 8) | ((unsigned)slot_of[2] << 16) | ((unsigned)slot_of[3] << 24);
-            packed.y = (unsigned)slot_of[4 % VEC] | ((unsigned)slot_of[5 % VEC] << 8) | ((unsigned)slot_of[6 % VEC] << 16) |
-                       ((unsigned)slot_of[7 % VEC] << 24);
-            *reinterpret_cast<uint2*>(arg + o) = packed;
-        } else {
-#pragma unroll
-            for (int i = 0; i < VEC; i++) arg[o + i] = (unsigned char)slot_of[i];
-        }
+        store_slots<VEC>(arg + o, slot_of);
     } else {
         if (OP == OP_AVG) {
             const float inv = 1.0f / (float)(g.J * g.T * g.R * g.S);
@@ -331,6 +397,97 @@ void pool_bprop_kernel(const T* __restrict__ E, const unsigned char* __restrict_
     store_vec<T, VEC>(B + ((long)c * per_map + inner) * VEC, acc);
 }
 
+// Backward for 2-D RS x RS windows of stride STR <= RS, known at compile time.
+// Shift the input by the padding and cut it into STR x STR cells: with
+// NW = ceil(RS / STR), every element of cell (cy,cx) is covered by windows out
+// of the same NW x NW, (cy-NW+1..cy) x (cx-NW+1..cx), and its tap inside each
+// of them is a compile-time constant.  One thread loads those errors (and
+// argmax bytes) once and produces the whole cell (3x3 /2: four windows for four
+// elements; 3x3 /1: nine for one; 2x2 /2: one for four), instead of every
+// element finding and decoding the windows of its own.  Accumulation order per
+// element is (p,q) ascending, as in pool_bprop_kernel.
+template <typename T, int VEC, int OP, int RS, int STR>
+__global__ __launch_bounds__(256)
+void pool_bprop_cell_kernel(const T* __restrict__ E, const unsigned char* __restrict__ arg, T* __restrict__ B, PoolGeom g)
+{
+    static_assert(VEC == 4 || VEC == 8, "one or two argmax words per packet");
+    static_assert(STR <= RS, "every element inside a window row / column range");
+    constexpr int NW = (RS + STR - 1) / STR;
+    typedef typename Pack<T, VEC>::raw_t raw_t;
+    const unsigned per_map = (unsigned)(g.D * g.cells_h * g.cells_w * g.nvec);
+    const unsigned inner = blockIdx.x * 256u + threadIdx.x;
+    int nv, cx, cy, z;
+    if (!split_inner(inner, per_map, g.div_nvec, g.div_cw, g.div_ch, g.nvec, g.cells_w, g.cells_h, nv, cx, cy, z)) return;
+    // one feature map holds fewer than 2^31 elements: 32-bit offsets inside it
+    const long out_map = (long)blockIdx.y * g.M * g.P * g.Q * g.N;
+    const T* Em = E + out_map;
+    const unsigned char* am = arg + (OP == OP_MAX ? out_map : 0);
+    T* Bm = B + (long)blockIdx.y * g.D * g.H * g.W * g.N;
+
+    raw_t eraw[NW * NW];
+    unsigned words[NW * NW][2];
+#pragma unroll
+    for (int w = 0; w < NW * NW; w++) {
+        const int p = cy - (NW - 1) + w / NW, q = cx - (NW - 1) + w % NW;
+        const bool ok = (unsigned)p < (unsigned)g.P && (unsigned)q < (unsigned)g.Q;
+        const unsigned o = ok ? (unsigned)((((z * g.P + p) * g.Q + q) * g.nvec + nv) * VEC) : (unsigned)(nv * VEC);
+        eraw[w] = load_packet(reinterpret_cast<const raw_t*>(Em + o));
+        if (OP == OP_MAX) {
+            // a window outside the output matches no tap
+            if (VEC == 8) {
+                const uint2 a = *reinterpret_cast<const uint2*>(am + o);
+                words[w][0] = ok ? a.x : 0xFFFFFFFFu;
+                words[w][1] = ok ? a.y : 0xFFFFFFFFu;
+            } else {
+                const unsigned a = *reinterpret_cast<const unsigned*>(am + o);
+                words[w][0] = words[w][1] = ok ? a : 0xFFFFFFFFu;
+            }
+        } else if (!ok) {
+            eraw[w] = raw_t{};
+        }
+    }
+
+    float acc[STR * STR][VEC];
+#pragma unroll
+    for (int px = 0; px < STR * STR; px++)
+#pragma unroll
+        for (int i = 0; i < VEC; i++) acc[px][i] = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW * NW; w++) {
+        const T* e = reinterpret_cast<const T*>(&eraw[w]);
+        float ev[VEC];
+        int   tap[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; i++) {
+            ev[i] = (float)e[i];
+            tap[i] = (int)((words[w][i >> 2] >> (8 * (i & 3))) & 0xFF);
+        }
+#pragma unroll
+        for (int px = 0; px < STR * STR; px++) {
+            // row / column of cell element px inside window w
+            const int ty = px / STR + (NW - 1 - w / NW) * STR, tx = px % STR + (NW - 1 - w % NW) * STR;
+            if (ty >= RS || tx >= RS) continue;
+#pragma unroll
+            for (int i = 0; i < VEC; i++) {
+                if (OP == OP_MAX) acc[px][i] += (tap[i] == ty * RS + tx) ? ev[i] : 0.0f;
+                else              acc[px][i] += ev[i];
+            }
+        }
+    }
+
+    const float inv = 1.0f / (float)(RS * RS);
+#pragma unroll
+    for (int px = 0; px < STR * STR; px++) {
+        const int y = cy * STR + px / STR - g.pad_h, x = cx * STR + px % STR - g.pad_w;
+        if ((unsigned)y >= (unsigned)g.H || (unsigned)x >= (unsigned)g.W) continue;
+        if (OP == OP_AVG) {
+#pragma unroll
+            for (int i = 0; i < VEC; i++) acc[px][i] *= inv;
+        }
+        store_vec<T, VEC>(Bm + (unsigned)((((z * g.H + y) * g.W + x) * g.nvec + nv) * VEC), acc[px]);
+    }
+}
+
 // windows that tile the input exactly (stride == window, no padding, extents
 // divisible): one thread owns a whole window and writes all of its grad_I
 // elements, so max bprop needs a single pass and no argmax scratch.
@@ -427,6 +584,11 @@ static PoolGeom make_geom(const ng_pool_params& p, int vec, size_t elem_bytes)
     const size_t in_bytes = (size_t)p.C * p.D * p.H * p.W * p.N * elem_bytes;
     g.stream_in = (disjoint && in_bytes > (256u << 20)) ? 1 : 0;
     g.xcd_remap = (!disjoint && (long)p.M * p.P * p.Q * g.nvec >= 16 * 256) ? 1 : 0;
+    g.use_cells = 0;
+    g.cells_h = (p.H - 1 + p.pad_h) / p.str_h + 1;
+    g.cells_w = (p.W - 1 + p.pad_w) / p.str_w + 1;
+    g.div_ch = FastDiv::make((unsigned)g.cells_h);
+    g.div_cw = FastDiv::make((unsigned)g.cells_w);
     return g;
 }
 
@@ -495,10 +657,36 @@ static bool two_window_cover(const ng_pool_params& p)
     return p.J == 1 && p.T == 1 && (p.R + p.str_h - 1) / p.str_h <= 2 && (p.S + p.str_w - 1) / p.str_w <= 2;
 }
 
+// 2-D square windows over whole feature maps with a (window, stride) pair the
+// cell kernel is compiled for: 0 = none, else RS * 16 + STR
+static int cell_shape(const ng_pool_params& p)
+{
+    const bool plane = p.J == 1 && p.T == 1 && p.str_j == 1 && p.str_d == 1 && p.pad_j == 0 && p.pad_d == 0 &&
+                       p.K == p.C && p.M == p.D && p.R == p.S && p.str_h == p.str_w && p.pad_h >= 0 && p.pad_w >= 0;
+    if (!plane) return 0;
+    const int shape = p.R * 16 + p.str_h;
+    return (shape == 0x32 || shape == 0x31 || shape == 0x22) ? shape : 0;
+}
+
 template <typename T, int VEC, int OP>
 static void launch_gather(const PoolGeom& g, bool win2, dim3 grid, const T* E, const unsigned char* arg, T* B,
                           hipStream_t st)
 {
+    if constexpr (VEC > 1) {
+        const dim3 cgrid = grid_for((long)g.D * g.cells_h * g.cells_w * g.nvec, g.C);
+        switch (g.use_cells) {
+        case 0x32:
+            hipLaunchKernelGGL((pool_bprop_cell_kernel<T, VEC, OP, 3, 2>), cgrid, dim3(256), 0, st, E, arg, B, g);
+            return;
+        case 0x31:
+            hipLaunchKernelGGL((pool_bprop_cell_kernel<T, VEC, OP, 3, 1>), cgrid, dim3(256), 0, st, E, arg, B, g);
+            return;
+        case 0x22:
+            hipLaunchKernelGGL((pool_bprop_cell_kernel<T, VEC, OP, 2, 2>), cgrid, dim3(256), 0, st, E, arg, B, g);
+            return;
+        default: break;
+        }
+    }
     if (win2 && VEC == 8)
         hipLaunchKernelGGL((pool_bprop_kernel<T, VEC, OP, true>), grid, dim3(256), 0, st, E, arg, B, g);
     else
@@ -514,6 +702,7 @@ static int run_bprop(const ng_pool_params& p, int op, const void* I, const void*
     const dim3 out_grid = grid_for((long)g.M * g.P * g.Q * g.nvec, g.K, g.xcd_remap);
     const dim3 in_grid = grid_for((long)g.D * g.H * g.W * g.nvec, g.C);
     const bool win2 = two_window_cover(p);
+    g.use_cells = cell_shape(p);
     if (op == OP_AVG) {
         launch_gather<T, VEC, OP_AVG>(g, win2, in_grid, (const T*)E, nullptr, (T*)B, st);
         NG_CHECK_LAUNCH("pool avg bprop");

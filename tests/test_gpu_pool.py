@@ -18,6 +18,9 @@ CASES = [
     (24, 9, 1, 6, 6, 3, 1, 1, 1, (0, 0, 0, 0), (3, 1, 1, 1)),        # maxout over feature maps only
     (12, 5, 1, 9, 9, 1, 1, 3, 3, (0, 0, 0, 0), (1, 1, 4, 4)),        # stride > window: uncovered inputs
     (4, 4, 1, 8, 8, 1, 1, 3, 3, (0, 0, 0, 0), (1, 1, 1, 1)),         # N not a multiple of 8 (scalar path)
+    (16, 3, 2, 12, 10, 1, 1, 3, 3, (0, 0, 0, 0), (1, 1, 2, 2)),      # 3x3/2 on even extents: last row / column uncovered
+    (8, 4, 1, 7, 9, 1, 1, 3, 3, (0, 0, 1, 1), (1, 1, 2, 2)),         # 3x3/2 padded, odd non-square extents
+    (4, 5, 1, 9, 11, 1, 1, 3, 3, (0, 0, 0, 1), (1, 1, 2, 2)),        # 3x3/2, four images: vector path only in fp32
 ]
 
 
