@@ -14,17 +14,18 @@
 
 namespace ng {
 
-// filter (C,TRS,K) -> per-class matrices [(tap,k)][Cpad], zero padded in c
+// filter (C,TRS,K) -> per-class matrices [(tap,k)][Cpad], zero padded in c and
+// in k (Kpad rows per tap)
 template <typename T>
-__global__ void filter_relayout_kernel(const T* F, T* out, const int* tap_dest, int C, int RST, int K, int Cpad)
+__global__ void filter_relayout_kernel(const T* F, T* out, const int* tap_dest, int C, int RST, int K, int Kpad, int Cpad)
 {
-    const long total = (long)RST * K * Cpad;
+    const long total = (long)RST * Kpad * Cpad;
     for (long e = (long)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (long)gridDim.x * blockDim.x) {
         const int c = (int)(e % Cpad);
         const long r = e / Cpad;
-        const int k = (int)(r % K);
-        const int trs = (int)(r / K);
-        const T v = (c < C) ? F[((long)c * RST + trs) * K + k] : (T)0;
+        const int k = (int)(r % Kpad);
+        const int trs = (int)(r / Kpad);
+        const T v = (c < C && k < K) ? F[((long)c * RST + trs) * K + k] : (T)0;
         out[((long)tap_dest[trs] + k) * Cpad + c] = v;
     }
 }
@@ -69,7 +70,7 @@ static int bprop_merged(const ConvPlan& pl, const T* Fm, const void* E, void* gr
     DenseLoader<T, MC, true> al{Fm, 0, pl.m_rpad, pl.m_rpad, J};
     const int nblk = BLOCKED ? p.K / BK : 1;
     GatherColsLoader<T, T, BLOCKED, BK> bl{(const T*)E, BLOCKED ? pl.d_merged_taps : pl.d_merged_flat, J, lat,
-                                           1, 1, 1, p.M, p.P, p.Q, MPQN, FastDiv::make((unsigned)nblk), nblk};
+                                           1, 1, 1, p.M, p.P, p.Q, MPQN, FastDiv::make((unsigned)nblk), nblk, p.K};
     MergedLatticeStoreEpilogue<T> epi{(T*)gradI, pl.m_rows, p.C, FastDiv::make((unsigned)p.C),
                                       FastDiv::make((unsigned)(p.str_h * p.str_w)), FastDiv::make((unsigned)p.str_w),
                                       (long)p.D * p.H * p.W * p.N, lat, p.str_d, p.str_h, p.str_w, p.D, p.H, p.W, alpha};
@@ -108,11 +109,11 @@ static int bprop_class(const ConvPlan& pl, const BpropClass& c, const T* Fs, con
     const int MPQN = p.M * p.P * p.Q * p.N;
     const PixelLattice lat = PixelLattice::make(p.N, ncols, c.nx, c.nx * c.ny);
     DenseLoader<T, MC, true> al{Fs + c.w_row * pl.Cpad, 0, pl.Cpad, pl.Cpad, c.J};
-    const int nblk = BLOCKED ? p.K / BK : 1;
+    const int nblk = BLOCKED ? pl.Kpad / BK : 1;
     GatherColsLoader<T, T, BLOCKED, BK> bl{(const T*)E,
                                            BLOCKED ? pl.d_bprop_taps + c.tap_offset : pl.d_bprop_flat + c.flat_offset,
                                            c.J, lat, 1, 1, 1, p.M, p.P, p.Q,
-                                           MPQN, FastDiv::make((unsigned)nblk), nblk};
+                                           MPQN, FastDiv::make((unsigned)nblk), nblk, p.K};
     const int k_tiles = cdiv(c.J, BK);
     const bool dense = (p.str_d == 1 && p.str_h == 1 && p.str_w == 1);
     if (dense) {
@@ -147,13 +148,13 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
                                   : run_bprop_merged<T, false>(pl, F, E, gradI, alpha, ws, stream);
     T* Fs = (T*)ws;
     {
-        const long total = (long)pl.RST * p.K * pl.Cpad;
+        const long total = (long)pl.RST * pl.Kpad * pl.Cpad;
         const int blocks = (int)std::min<long>((total + 255) / 256, 4096);
         hipLaunchKernelGGL(filter_relayout_kernel<T>, dim3(blocks), dim3(256), 0, stream,
-                           (const T*)F, Fs, pl.d_tap_dest, p.C, pl.RST, p.K, pl.Cpad);
+                           (const T*)F, Fs, pl.d_tap_dest, p.C, pl.RST, p.K, pl.Kpad, pl.Cpad);
         NG_CHECK_LAUNCH("filter relayout");
     }
-    const bool blocked = p.K % pl.bk == 0;
+    const bool blocked = pl.bprop_blocked;
     for (const BpropClass& c : pl.classes) {
         if (c.nz * c.ny * c.nx == 0) continue;
         int rc;

@@ -15,17 +15,17 @@ static int fprop_tile(const ConvPlan& pl, const void* I, const void* F, void* O,
                               (flags & NG_FLAG_RELU) ? 1u : 0u, 0u, 0u, 0u, 1u};
     const PixelLattice lat = PixelLattice::make(p.N, ncols, p.Q, p.P * p.Q);
     if (BLOCKED) {
-        const int nblk = p.C / BK;
-        FilterBlockLoader<T, BK> al{(const T*)F, p.K, pl.RST * p.K, FastDiv::make((unsigned)nblk), nblk};
+        const int nblk = cdiv(p.C, BK);
+        FilterBlockLoader<T, BK> al{(const T*)F, p.K, pl.RST * p.K, FastDiv::make((unsigned)nblk), nblk, p.C};
         GatherColsLoader<T, TIN, true, BK> bl{(const TIN*)I, pl.d_fprop_taps, pl.CRST, lat,
                                               p.str_d, p.str_h, p.str_w, p.D, p.H, p.W,
-                                              DHWN, FastDiv::make((unsigned)nblk), nblk};
+                                              DHWN, FastDiv::make((unsigned)nblk), nblk, p.C};
         return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, epi, p.K, ncols, pl.RST * nblk, 1, stream, "conv fprop");
     } else {
         DenseLoader<T, MC, true> al{(const T*)F, 0, p.K, p.K, pl.CRST};
         GatherColsLoader<T, TIN, false, BK> bl{(const TIN*)I, pl.d_fprop_flat, pl.CRST, lat,
                                                p.str_d, p.str_h, p.str_w, p.D, p.H, p.W,
-                                               0, FastDiv{0, 0}, 1};
+                                               0, FastDiv{0, 0}, 1, 0};
         return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, epi, p.K, ncols, cdiv(pl.CRST, BK), 1, stream, "conv fprop");
     }
 }
@@ -59,7 +59,7 @@ extern "C" int ng_conv_fprop(const void* plan, int in_dtype, const void* I, cons
     int rc;
     if ((rc = check_ptr16(I, "I")) || (rc = check_ptr16(F, "F")) || (rc = check_ptr16(O, "O"))) return rc;
     hipStream_t st = (hipStream_t)stream;
-    const bool blocked = pl->p.C % pl->bk == 0;
+    const bool blocked = pl->fprop_blocked;
     if (pl->dtype == NG_F16) {
         if (in_dtype == NG_F16)
             return blocked ? fprop_h<_Float16, true>(*pl, I, F, O, alpha, flags, st)

@@ -120,12 +120,14 @@ struct GatherColsLoader {
     int             row_stride; // BLOCKED: elements between consecutive rows of a block
     FastDiv         blk_div;    // BLOCKED: tile index -> tap (blocks per tap = nblk)
     int             nblk;
+    int             chan;       // BLOCKED: rows per tap; the last block of a tap may be partly empty
 
     // same-type inputs are plain 16-byte buffer loads (see DenseLoader::DIRECT)
     static constexpr bool DIRECT = std::is_same<T, TIN>::value;
     static constexpr bool TILE_READS_TABLE = BLOCKED;
 
     struct Ctx { int base, z0, y0, x0, kr; };
+    // k0: flat: first contraction row of the tile; BLOCKED: rows of the block that exist
     struct Tile { BufferRsrc rsrc; int toff, dz, dy, dx, k0; };
 
     __device__ __forceinline__ Ctx prepare(int col, int kr) const
@@ -152,6 +154,7 @@ struct GatherColsLoader {
             const TapEntry e = tab[tap];
             t.toff = e.off + blk * BK * row_stride;
             t.dz = e.dz; t.dy = e.dy; t.dx = e.dx;
+            t.k0 = chan - blk * BK;
         } else {
             t.toff = 0; t.dz = t.dy = t.dx = 0;
         }
@@ -164,7 +167,7 @@ struct GatherColsLoader {
         constexpr int ES = ChunkFetch<T, TIN>::ES;
         if (BLOCKED) {
             const bool ok = (unsigned)(c.z0 + t.dz) < (unsigned)lim_d && (unsigned)(c.y0 + t.dy) < (unsigned)lim_h &&
-                            (unsigned)(c.x0 + t.dx) < (unsigned)lim_w;
+                            (unsigned)(c.x0 + t.dx) < (unsigned)lim_w && c.kr < t.k0;
             return ok ? (unsigned)(c.base + t.toff) * ES : NG_OOB_OFFSET;
         } else {
             const int k = t.k0 + c.kr;
@@ -183,7 +186,8 @@ struct GatherColsLoader {
 
 // A operand of blocked fprop: filter F[c][tap][k] read as rows j = (tap, c):
 // tile (tap, block) holds channels block*BK .. +BK-1, consecutive rows are
-// RST*K elements apart.
+// RST*K elements apart.  The last block of a tap may reach past channel C-1:
+// those rows are not read (zero operands).
 template <typename T, int BK>
 struct FilterBlockLoader {
     const T* F;
@@ -191,17 +195,19 @@ struct FilterBlockLoader {
     int      RSTK;       // elements between consecutive channels
     FastDiv  blk_div;
     int      nblk;
+    int      C;          // channels
 
     static constexpr bool DIRECT = true;
     static constexpr bool TILE_READS_TABLE = false;
 
-    struct Ctx { unsigned off; };
-    struct Tile { BufferRsrc rsrc; };
+    struct Ctx { unsigned off; int kr; };
+    struct Tile { BufferRsrc rsrc; int rows; };
 
     __device__ __forceinline__ Ctx prepare(int m, int kr) const
     {
         Ctx c;
         c.off = (m < K) ? (unsigned)(kr * RSTK + m) * (unsigned)sizeof(T) : NG_OOB_OFFSET;
+        c.kr = kr;
         return c;
     }
     __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/) const
@@ -210,10 +216,14 @@ struct FilterBlockLoader {
         const int blk = kt - tap * nblk;
         Tile t;
         t.rsrc = make_rsrc(F + (long)blk * BK * RSTK + (long)tap * K);
+        t.rows = C - blk * BK;
         return t;
     }
-    __device__ __forceinline__ unsigned offset(const Tile& /*t*/, const Ctx& c) const { return c.off; }
-    __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const { return buffer_load_chunk(t.rsrc, c.off); }
+    __device__ __forceinline__ unsigned offset(const Tile& t, const Ctx& c) const
+    {
+        return c.kr < t.rows ? c.off : NG_OOB_OFFSET;
+    }
+    __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const { return buffer_load_chunk(t.rsrc, offset(t, c)); }
 };
 
 // A operand of update (contraction-contiguous tile: rows are filter rows

@@ -24,6 +24,11 @@ struct ConvPlan {
     int dtype;
     int bk;                 // contraction tile depth of the kernels for this dtype
     int CRST, RST, Cpad;
+    // Blocked contraction tiles (one filter tap x bk channels) are used when the
+    // channel count is a multiple of bk or padding it to one wastes little;
+    // Kpad is K rounded up to bk when the data gradient runs blocked, else K.
+    bool fprop_blocked = false, bprop_blocked = false;
+    int Kpad = 0;
     TapEntry* d_fprop_flat = nullptr;   // CRST entries, rows (c,t,r,s)
     TapEntry* d_fprop_taps = nullptr;   // RST entries
     TapEntry* d_bprop_flat = nullptr;   // K*RST entries grouped by class, rows (tap,k)
@@ -43,6 +48,9 @@ struct ConvPlan {
 };
 
 inline int cdiv(int a, int b) { return (a + b - 1) / b; }
+
+// channel blocks of depth bk: exact, or padded by at most one half
+inline bool blocks_pay(int channels, int bk) { return channels % bk == 0 || 2 * cdiv(channels, bk) * bk <= 3 * channels; }
 
 // how many slices to cut a contraction into so that the grid fills the chip
 inline int conv_splits(int out_tiles, int total_k_tiles, size_t slice_bytes, size_t ws_bytes)

@@ -27,6 +27,9 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
     pl->RST = p.T * p.R * p.S;
     pl->CRST = p.C * pl->RST;
     pl->Cpad = cdiv(p.C, 8) * 8;
+    pl->fprop_blocked = blocks_pay(p.C, pl->bk);
+    pl->bprop_blocked = blocks_pay(p.K, pl->bk);
+    pl->Kpad = pl->bprop_blocked ? cdiv(p.K, pl->bk) * pl->bk : p.K;
     const int HW = p.H * p.W, DHW = p.D * HW;
 
     // forward taps
@@ -68,7 +71,7 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
                             if ((rx + p.pad_w - s) % p.str_w) continue;
                             const int dz = (rz + p.pad_d - t) / p.str_d, dy = (ry + p.pad_h - r) / p.str_h,
                                       dx = (rx + p.pad_w - s) / p.str_w;
-                            tap_dest[(size_t)(t * p.R + r) * p.S + s] = (int)(w_row + (long)taps * p.K);
+                            tap_dest[(size_t)(t * p.R + r) * p.S + s] = (int)(w_row + (long)taps * pl->Kpad);
                             btaps.push_back(TapEntry{(int)(((long)dz * PQ + dy * p.Q + dx) * p.N), dz, dy, dx});
                             for (int k = 0; k < p.K; k++)
                                 bflat.push_back(TapEntry{(int)(((long)k * p.M * PQ + (long)dz * PQ + dy * p.Q + dx) * p.N),
@@ -78,7 +81,7 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
                     }
                 }
                 c.taps = taps;
-                c.J = taps * p.K;
+                c.J = taps * pl->Kpad;
                 w_row += c.J;
                 pl->classes.push_back(c);
             }
@@ -126,7 +129,7 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
     if (!rc) rc = upload(mflat.data(), mflat.size() * sizeof(TapEntry), (void**)&pl->d_merged_flat);
     if (rc) { ng_conv_plan_destroy(pl); return rc; }
 
-    pl->ws_bprop = align_up((size_t)pl->RST * p.K * pl->Cpad * dtype_size(dtype), 256);
+    pl->ws_bprop = align_up((size_t)pl->RST * pl->Kpad * pl->Cpad * dtype_size(dtype), 256);
     if (pl->merged)
         pl->ws_bprop = std::max(pl->ws_bprop, align_up((size_t)pl->m_taps * p.K * pl->m_rpad * dtype_size(dtype), 256));
     {

@@ -20,6 +20,11 @@ SMALL = [
     (64, 8, 8, 1, 7, 7, 1, 1, 1, (0, 0, 0), (1, 1, 1)),           # 1x1
     (8, 20, 24, 1, 12, 12, 1, 2, 2, (0, 0, 0), (1, 3, 3)),        # stride > filter: unreached input pixels
     (8, 72, 64, 1, 12, 11, 1, 3, 3, (0, 1, 1), (1, 2, 2)),        # strided, classes * C > 256: one launch per class
+    # channel counts that are not multiples of the contraction tile: blocks padded with unread rows
+    (16, 96, 112, 1, 9, 9, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (16, 144, 48, 1, 7, 7, 1, 1, 1, (0, 0, 0), (1, 1, 1)),        # 1x1 (inception style)
+    (8, 96, 112, 1, 11, 10, 1, 3, 3, (0, 1, 1), (1, 2, 2)),       # strided, one launch per class
+    (8, 48, 208, 1, 6, 6, 1, 2, 2, (0, 1, 1), (1, 1, 1)),
 ]
 
 
