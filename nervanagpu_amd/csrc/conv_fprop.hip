@@ -37,11 +37,10 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
     case 256: return fprop_tile<_Float16, TIN, BLOCKED, 256, 256, 64, 2, 4>(pl, I, F, O, alpha, flags, st);
     case 128: return fprop_tile<_Float16, TIN, BLOCKED, 128, 256, 64, 1, 4>(pl, I, F, O, alpha, flags, st);
     default:
-        // a first layer's whole contraction (C*T*R*S <= 32) fits a half-depth
-        // tile: half the LDS, twice the workgroups per CU for a kernel that is
-        // all prologue and epilogue
-        if (!BLOCKED && pl.CRST <= 32)
-            return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 32, 1, 4>(pl, I, F, O, alpha, flags, st);
+        // Row-by-row gathered contractions (first layers, few channels) are bound
+        // by request latency, not by the matrix pipe: half-depth tiles halve the
+        // LDS footprint, so twice as many workgroups per CU keep requests in flight
+        if (!BLOCKED) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 32, 1, 4>(pl, I, F, O, alpha, flags, st);
         return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 64, 1, 4>(pl, I, F, O, alpha, flags, st);
     }
 }
