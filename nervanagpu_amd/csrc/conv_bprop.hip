@@ -92,7 +92,7 @@ static int run_bprop_merged(const ConvPlan& pl, const void* F, const void* E, vo
     if constexpr (sizeof(T) == 2) {
         switch (pick_row_tile(pl.m_rows, pl.m_nz * pl.m_ny * pl.m_nx * p.N, 256)) {
         case 256: return bprop_merged<T, BLOCKED, 256, 256, 64, 2, 4>(pl, Fm, E, gradI, alpha, stream);
-        case 128: return bprop_merged<T, BLOCKED, 128, 256, 64, 1, 4>(pl, Fm, E, gradI, alpha, stream);
+        case 128: return bprop_merged<T, BLOCKED, 128, 256, 64, 2, 4>(pl, Fm, E, gradI, alpha, stream);
         default:  return bprop_merged<T, BLOCKED, 64, 256, 64, 1, 4>(pl, Fm, E, gradI, alpha, stream);
         }
     } else {
@@ -131,7 +131,7 @@ static int bprop_class_h(const ConvPlan& pl, const BpropClass& c, const _Float16
 {
     switch (pick_row_tile(pl.p.C, c.nz * c.ny * c.nx * pl.p.N, 256)) {
     case 256: return bprop_class<_Float16, BLOCKED, 256, 256, 64, 2, 4>(pl, c, Fs, E, gradI, alpha, st);
-    case 128: return bprop_class<_Float16, BLOCKED, 128, 256, 64, 1, 4>(pl, c, Fs, E, gradI, alpha, st);
+    case 128: return bprop_class<_Float16, BLOCKED, 128, 256, 64, 2, 4>(pl, c, Fs, E, gradI, alpha, st);
     default:  return bprop_class<_Float16, BLOCKED, 64, 256, 64, 1, 4>(pl, c, Fs, E, gradI, alpha, st);
     }
 }

@@ -35,7 +35,9 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
 {
     switch (pick_row_tile(pl.p.K, pl.p.M * pl.p.P * pl.p.Q * pl.p.N, 256)) {
     case 256: return fprop_tile<_Float16, TIN, BLOCKED, 256, 256, 64, 2, 4>(pl, I, F, O, alpha, flags, st);
-    case 128: return fprop_tile<_Float16, TIN, BLOCKED, 128, 256, 64, 1, 4>(pl, I, F, O, alpha, flags, st);
+    // 128 rows on eight wavefronts: mid-sized layers run about one workgroup per
+    // CU, and twice the wavefronts hide the LDS and request latency of a tile
+    case 128: return fprop_tile<_Float16, TIN, BLOCKED, 128, 256, 64, 2, 4>(pl, I, F, O, alpha, flags, st);
     default:
         // Row-by-row gathered contractions (first layers, few channels) are bound
         // by request latency, not by the matrix pipe: half-depth tiles halve the
