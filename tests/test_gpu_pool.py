@@ -69,6 +69,34 @@ def test_max_pool_ties_and_out_of_bounds(ng):
     assert np.array_equal(dB.get(), ref.astype(np.float16))
 
 
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_max_pool_negative_inputs_padding_and_signed_zero_ties(ng, dtype):
+    """padding never wins a window (all inputs negative), and among +0 / -0 ties the
+    first element in scan order receives the error (numeric, not bitwise, equality)"""
+    rng = np.random.default_rng(12)
+    for (N, C, H, W, R, pad, strd) in ((16, 6, 9, 10, 3, 1, 2), (16, 4, 8, 8, 2, 1, 2), (8, 5, 7, 7, 3, 1, 1)):
+        layer = ng.pool_layer(dtype, "max", N, C, 1, H, W, 1, 1, R, R, 0, 0, pad, pad, 1, 1, strd, strd)
+        I = rng.uniform(-2, -1, layer.dimI).astype(dtype)
+        E = rng.uniform(-1, 1, layer.dimO).astype(dtype)
+        for variant in ("negative", "zeros"):
+            if variant == "zeros":
+                # non-positive data with many exact zeros of both signs: windows tie on zero
+                I = np.where(rng.random(layer.dimI) < 0.5, 0.0, I).astype(dtype)
+                I[(I == 0) & (rng.random(layer.dimI) < 0.5)] = -0.0
+                assert np.signbit(I[I == 0]).any() and (~np.signbit(I[I == 0])).any()
+            dI, dE = ng.array(I, dtype=dtype), ng.array(E, dtype=dtype)
+            dO, dB = ng.empty(layer.dimO, dtype=dtype), ng.empty(layer.dimI, dtype=dtype)
+            ng.fprop_pool(layer, dI, dO)
+            ng.bprop_pool(layer, dI, dE, dB)
+            refO = orc.ref_pool_fprop(I, "max", layer.JTRS, layer.padding, layer.strides)
+            refB = orc.ref_pool_bprop(I, E, "max", layer.JTRS, layer.padding, layer.strides)
+            assert np.array_equal(dO.get(), refO.astype(dtype)), variant
+            if dtype == np.float16:
+                assert_fp16_within_ulp(dB.get(), refB, 1.0, "max bprop " + variant, 1e-6)
+            else:
+                np.testing.assert_allclose(dB.get(), refB, rtol=1e-5, atol=1e-6)
+
+
 def test_config4_vgg_pool_shapes(ng):
     """2x2/2 max pooling at the five block ends of config 4 (reduced in C to bound
     host time, full in H, W, N); idempotent structure: pooled gradient sums match"""
