@@ -72,20 +72,27 @@ inline int check_ptr16(const void* p, const char* what)
 }
 
 // Row tile (output feature maps or input channels) for BN-column tiles: the
-// candidate with the least estimated time, rounds of workgroups over the chip
-// times the work of one workgroup, where the 256-row tile runs about a third
-// more efficiently than the narrower ones (measured on dense problems).
-// Padding rows count as work, so a 64-row problem picks the 64-row tile.
+// candidate with the least estimated time per contraction tile, rounds of
+// workgroups over the chip times the duration of one tile step of that shape.
+// The steps are measured ones (microseconds per 64-deep tile with the CU to
+// itself: 256 rows and 128 rows on eight wavefronts, 64 rows on four); two
+// 64-row workgroups fit the LDS of a CU and overlap, the larger shapes run one
+// per CU.  Padding rows count as work through the number of row tiles, so a
+// 64-row problem with many column tiles picks the 64-row tile, while a grid of
+// at most one workgroup per CU prefers the 128-row tile, whose eight wavefronts
+// hide the latency of a tile step better.
 inline int pick_row_tile(int rows, int ncols, int bn)
 {
     static const int tiles[3] = {256, 128, 64};
-    static const double eff[3] = {1.0, 0.75, 0.75};
+    static const int resident[3] = {1, 1, 2};
+    static const double step_us[3] = {1.95, 1.2, 1.39};
     const int cus = device_cu_count();
     int best = tiles[0];
     double best_cost = 0.0;
     for (int i = 0; i < 3; i++) {
         const long blocks = (long)cdiv(rows, tiles[i]) * cdiv(ncols, bn);
-        const double cost = (double)((blocks + cus - 1) / cus) * tiles[i] / eff[i];
+        const long slots = (long)cus * resident[i];
+        const double cost = (double)((blocks + slots - 1) / slots) * step_us[i];
         if (i == 0 || cost < best_cost * 0.999) { best = tiles[i]; best_cost = cost; }
     }
     return best;
