@@ -91,7 +91,7 @@ inline int pick_row_tile(int rows, int ncols, int bn)
 {
     static const int tiles[3] = {256, 128, 64};
     static const int resident[3] = {1, 1, 2};
-    static const double step_us[3] = {1.95, 1.2, 1.39};
+    static const double step_us[3] = {1.75, 1.2, 1.39};
     const int cus = device_cu_count();
     int best = tiles[0];
     double best_cost = 0.0;
