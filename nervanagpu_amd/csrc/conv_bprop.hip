@@ -2,7 +2,10 @@
 // Replaces {h,s}conv_bprop_{C64_N64,C32_N64} and the dimShuffle / transpose /
 // memset launches around them (nervanagpu/nervanagpu.py:652-659, 685-719).
 //
-// Always the gather form, for every C and stride: strided layers are decomposed
+// Always the gather form, for every C and stride.  The filter operand is read
+// in place (rows c, contraction (tap, k), k contiguous per tap) whenever the
+// contraction runs in blocks of output maps; the row-by-row form for few output
+// maps first re-lays the filter out into [(tap,k)][C].  Strided layers are decomposed
 // into str_d*str_h*str_w stride-1 sub-problems (one per residue class of the
 // input pixel), each with only the taps that can reach that class.  When all
 // classes together have at most 256 rows (few channels, e.g. a first layer)
@@ -101,14 +104,13 @@ static int run_bprop_merged(const ConvPlan& pl, const void* F, const void* E, vo
 }
 
 template <typename T, bool BLOCKED, int BM, int BN, int BK, int WM, int WN>
-static int bprop_class(const ConvPlan& pl, const BpropClass& c, const T* Fs, const void* E, void* gradI,
+static int bprop_class(const ConvPlan& pl, const BpropClass& c, const void* F, const T* Fs, const void* E, void* gradI,
                        float alpha, hipStream_t stream)
 {
     const ng_conv_params& p = pl.p;
     const int ncols = c.nz * c.ny * c.nx * p.N;
     const int MPQN = p.M * p.P * p.Q * p.N;
     const PixelLattice lat = PixelLattice::make(p.N, ncols, c.nx, c.nx * c.ny);
-    DenseLoader<T, MC, true> al{Fs + c.w_row * pl.Cpad, 0, pl.Cpad, pl.Cpad, c.J};
     const int nblk = BLOCKED ? pl.Kpad / BK : 1;
     GatherColsLoader<T, T, BLOCKED, BK> bl{(const T*)E,
                                            BLOCKED ? pl.d_bprop_taps + c.tap_offset : pl.d_bprop_flat + c.flat_offset,
@@ -116,23 +118,30 @@ static int bprop_class(const ConvPlan& pl, const BpropClass& c, const T* Fs, con
                                            MPQN, FastDiv::make((unsigned)nblk), nblk, p.K};
     const int k_tiles = cdiv(c.J, BK);
     const bool dense = (p.str_d == 1 && p.str_h == 1 && p.str_w == 1);
-    if (dense) {
-        ScaleStoreEpilogue<T> epi{(T*)gradI, 0, ncols, p.C, ncols, alpha, 0.0f, 0u, 0u, 0u, 0u, 1u};
-        return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, epi, p.C, ncols, k_tiles, 1, stream, "conv bprop");
+    ScaleStoreEpilogue<T> depi{(T*)gradI, 0, ncols, p.C, ncols, alpha, 0.0f, 0u, 0u, 0u, 0u, 1u};
+    LatticeStoreEpilogue<T> lepi{(T*)gradI, p.C, (long)p.D * p.H * p.W * p.N, lat, c.rz, c.ry, c.rx,
+                                 p.str_d, p.str_h, p.str_w, p.H, p.W, alpha};
+    if constexpr (BLOCKED) {
+        // the filter is read in place: rows c, contraction (tap, k)
+        FilterRowsLoader<T, BK> al{(const T*)F, pl.d_bprop_trs + c.tap_offset, p.C, p.K, pl.RST * p.K,
+                                   FastDiv::make((unsigned)nblk), nblk};
+        if (dense) return launch_core<T, BM, BN, BK, WM, WN, KC, MC>(al, bl, depi, p.C, ncols, k_tiles, 1, stream, "conv bprop");
+        return launch_core<T, BM, BN, BK, WM, WN, KC, MC>(al, bl, lepi, p.C, ncols, k_tiles, 1, stream, "conv bprop");
+    } else {
+        DenseLoader<T, MC, true> al{Fs + c.w_row * pl.Cpad, 0, pl.Cpad, pl.Cpad, c.J};
+        if (dense) return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, depi, p.C, ncols, k_tiles, 1, stream, "conv bprop");
+        return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, lepi, p.C, ncols, k_tiles, 1, stream, "conv bprop");
     }
-    LatticeStoreEpilogue<T> epi{(T*)gradI, p.C, (long)p.D * p.H * p.W * p.N, lat, c.rz, c.ry, c.rx,
-                                p.str_d, p.str_h, p.str_w, p.H, p.W, alpha};
-    return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, epi, p.C, ncols, k_tiles, 1, stream, "conv bprop");
 }
 
 template <bool BLOCKED>
-static int bprop_class_h(const ConvPlan& pl, const BpropClass& c, const _Float16* Fs, const void* E, void* gradI,
-                         float alpha, hipStream_t st)
+static int bprop_class_h(const ConvPlan& pl, const BpropClass& c, const void* F, const _Float16* Fs, const void* E,
+                         void* gradI, float alpha, hipStream_t st)
 {
     switch (pick_row_tile(pl.p.C, c.nz * c.ny * c.nx * pl.p.N, 256)) {
-    case 256: return bprop_class<_Float16, BLOCKED, 256, 256, 64, 2, 4>(pl, c, Fs, E, gradI, alpha, st);
-    case 128: return bprop_class<_Float16, BLOCKED, 128, 256, 64, 2, 4>(pl, c, Fs, E, gradI, alpha, st);
-    default:  return bprop_class<_Float16, BLOCKED, 64, 256, 64, 1, 4>(pl, c, Fs, E, gradI, alpha, st);
+    case 256: return bprop_class<_Float16, BLOCKED, 256, 256, 64, 2, 4>(pl, c, F, Fs, E, gradI, alpha, st);
+    case 128: return bprop_class<_Float16, BLOCKED, 128, 256, 64, 2, 4>(pl, c, F, Fs, E, gradI, alpha, st);
+    default:  return bprop_class<_Float16, BLOCKED, 64, 256, 64, 1, 4>(pl, c, F, Fs, E, gradI, alpha, st);
     }
 }
 
@@ -147,23 +156,23 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
         return (p.K % pl.bk == 0) ? run_bprop_merged<T, true>(pl, F, E, gradI, alpha, ws, stream)
                                   : run_bprop_merged<T, false>(pl, F, E, gradI, alpha, ws, stream);
     T* Fs = (T*)ws;
-    {
+    const bool blocked = pl.bprop_blocked;
+    if (!blocked) {
         const long total = (long)pl.RST * pl.Kpad * pl.Cpad;
         const int blocks = (int)std::min<long>((total + 255) / 256, 4096);
         hipLaunchKernelGGL(filter_relayout_kernel<T>, dim3(blocks), dim3(256), 0, stream,
                            (const T*)F, Fs, pl.d_tap_dest, p.C, pl.RST, p.K, pl.Kpad, pl.Cpad);
         NG_CHECK_LAUNCH("filter relayout");
     }
-    const bool blocked = pl.bprop_blocked;
     for (const BpropClass& c : pl.classes) {
         if (c.nz * c.ny * c.nx == 0) continue;
         int rc;
         if (sizeof(T) == 2)
-            rc = blocked ? bprop_class_h<true>(pl, c, (const _Float16*)Fs, E, gradI, alpha, stream)
-                         : bprop_class_h<false>(pl, c, (const _Float16*)Fs, E, gradI, alpha, stream);
+            rc = blocked ? bprop_class_h<true>(pl, c, F, (const _Float16*)Fs, E, gradI, alpha, stream)
+                         : bprop_class_h<false>(pl, c, F, (const _Float16*)Fs, E, gradI, alpha, stream);
         else
-            rc = blocked ? bprop_class<float, true, 128, 128, 16, 2, 2>(pl, c, (const float*)Fs, E, gradI, alpha, stream)
-                         : bprop_class<float, false, 128, 128, 16, 2, 2>(pl, c, (const float*)Fs, E, gradI, alpha, stream);
+            rc = blocked ? bprop_class<float, true, 128, 128, 16, 2, 2>(pl, c, F, (const float*)Fs, E, gradI, alpha, stream)
+                         : bprop_class<float, false, 128, 128, 16, 2, 2>(pl, c, F, (const float*)Fs, E, gradI, alpha, stream);
         if (rc) return rc;
     }
     return 0;

@@ -226,6 +226,54 @@ struct FilterBlockLoader {
     __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const { return buffer_load_chunk(t.rsrc, offset(t, c)); }
 };
 
+// A operand of the blocked data gradient: the filter F[c][trs][k] in place,
+// read as rows c with the contraction (tap, k): for one tap the k values of a
+// row are contiguous, so tile (tap, block) is a contraction-contiguous tile of
+// rows RST*K elements apart starting at trs(tap)*K + block*BK.  The taps of a
+// residue class come from a small table (filter position of each class tap);
+// the last block of a tap may reach past k = K-1: those chunks are not read.
+template <typename T, int BK>
+struct FilterRowsLoader {
+    const T*   F;
+    const int* tap_trs;   // filter position (t*R + r)*S + s of each tap of the class
+    int        C;         // rows
+    int        K;         // contraction extent per tap
+    int        RSTK;      // elements between consecutive rows
+    FastDiv    blk_div;   // tile index -> tap (blocks per tap = nblk)
+    int        nblk;
+
+    static constexpr bool DIRECT = true;
+    static constexpr bool TILE_READS_TABLE = true;
+
+    struct Ctx { unsigned off; int kc; };
+    struct Tile { BufferRsrc rsrc; int kvalid; };
+
+    __device__ __forceinline__ Ctx prepare(int row, int kc) const
+    {
+        Ctx c;
+        c.kc = kc;
+        c.off = (row < C) ? ((unsigned)row * (unsigned)RSTK + (unsigned)kc) * (unsigned)sizeof(T) : NG_OOB_OFFSET;
+        return c;
+    }
+    __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/) const
+    {
+        const int tap = (int)blk_div.div((unsigned)kt);
+        const int blk = kt - tap * nblk;
+        Tile t;
+        // the table entry is wavefront-uniform; the descriptor must live in scalar registers
+        const int trs = __builtin_amdgcn_readfirstlane(tap_trs[tap]);
+        t.rsrc = make_rsrc(F + (long)trs * K + (long)blk * BK);
+        t.kvalid = K - blk * BK;
+        return t;
+    }
+    // K is a multiple of the chunk length, so a chunk is inside or outside as a whole
+    __device__ __forceinline__ unsigned offset(const Tile& t, const Ctx& c) const
+    {
+        return c.kc < t.kvalid ? c.off : NG_OOB_OFFSET;
+    }
+    __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const { return buffer_load_chunk(t.rsrc, offset(t, c)); }
+};
+
 // A operand of update (contraction-contiguous tile: rows are filter rows
 // j = (c,t,r,s), the contraction index is (output pixel, n)).  BLOCKED: N is a
 // multiple of BK, so a tile lies inside one output pixel.

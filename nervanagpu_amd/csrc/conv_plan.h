@@ -33,6 +33,7 @@ struct ConvPlan {
     TapEntry* d_fprop_taps = nullptr;   // RST entries
     TapEntry* d_bprop_flat = nullptr;   // K*RST entries grouped by class, rows (tap,k)
     TapEntry* d_bprop_taps = nullptr;   // RST entries grouped by class
+    int* d_bprop_trs = nullptr;         // RST ints grouped by class: filter position of each class tap
     int* d_tap_dest = nullptr;          // RST ints: first re-laid filter row of each tap
     std::vector<BpropClass> classes;
     // Merged form of the strided data gradient (used when all classes together

@@ -48,6 +48,7 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
     // data-gradient classes: input pixel (z,y,x) with z % str_d == rz ... receives
     // tap t iff (rz + pad_d - t) % str_d == 0, from output m = iz + (rz + pad_d - t)/str_d
     std::vector<TapEntry> bflat, btaps;
+    std::vector<int> btrs;
     std::vector<int> tap_dest((size_t)pl->RST, 0);
     const int PQ = p.P * p.Q;
     long w_row = 0;
@@ -73,6 +74,7 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
                                       dx = (rx + p.pad_w - s) / p.str_w;
                             tap_dest[(size_t)(t * p.R + r) * p.S + s] = (int)(w_row + (long)taps * pl->Kpad);
                             btaps.push_back(TapEntry{(int)(((long)dz * PQ + dy * p.Q + dx) * p.N), dz, dy, dx});
+                            btrs.push_back((t * p.R + r) * p.S + s);
                             for (int k = 0; k < p.K; k++)
                                 bflat.push_back(TapEntry{(int)(((long)k * p.M * PQ + (long)dz * PQ + dy * p.Q + dx) * p.N),
                                                          dz, dy, dx});
@@ -124,6 +126,7 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
     if (!rc) rc = upload(ftaps.data(), ftaps.size() * sizeof(TapEntry), (void**)&pl->d_fprop_taps);
     if (!rc) rc = upload(bflat.data(), bflat.size() * sizeof(TapEntry), (void**)&pl->d_bprop_flat);
     if (!rc) rc = upload(btaps.data(), btaps.size() * sizeof(TapEntry), (void**)&pl->d_bprop_taps);
+    if (!rc) rc = upload(btrs.data(), btrs.size() * sizeof(int), (void**)&pl->d_bprop_trs);
     if (!rc) rc = upload(tap_dest.data(), tap_dest.size() * sizeof(int), (void**)&pl->d_tap_dest);
     if (!rc) rc = upload(mtaps.data(), mtaps.size() * sizeof(TapEntry), (void**)&pl->d_merged_taps);
     if (!rc) rc = upload(mflat.data(), mflat.size() * sizeof(TapEntry), (void**)&pl->d_merged_flat);
@@ -151,6 +154,7 @@ int ng_conv_plan_destroy(void* plan)
     if (pl->d_fprop_taps) (void)hipFree(pl->d_fprop_taps);
     if (pl->d_bprop_flat) (void)hipFree(pl->d_bprop_flat);
     if (pl->d_bprop_taps) (void)hipFree(pl->d_bprop_taps);
+    if (pl->d_bprop_trs) (void)hipFree(pl->d_bprop_trs);
     if (pl->d_tap_dest) (void)hipFree(pl->d_tap_dest);
     if (pl->d_merged_taps) (void)hipFree(pl->d_merged_taps);
     if (pl->d_merged_flat) (void)hipFree(pl->d_merged_flat);
