@@ -150,7 +150,7 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
                      void* ws, size_t ws_bytes, hipStream_t stream)
 {
     const ng_conv_params& p = pl.p;
-    if (ws_bytes < pl.ws_bprop || !ws)
+    if (pl.ws_bprop && (ws_bytes < pl.ws_bprop || !ws))
         return fail(-40, "ng_conv_bprop: workspace too small (%zu < %zu)", ws_bytes, pl.ws_bprop);
     if (pl.merged)
         return (p.K % pl.bk == 0) ? run_bprop_merged<T, true>(pl, F, E, gradI, alpha, ws, stream)
@@ -189,7 +189,7 @@ extern "C" int ng_conv_bprop(const void* plan, const void* F, const void* E, voi
     if (!pl) return fail(-48, "conv: null plan");
     int rc;
     if ((rc = check_ptr16(F, "F")) || (rc = check_ptr16(E, "E")) || (rc = check_ptr16(gradI, "grad_I")) ||
-        (rc = check_ptr16(workspace, "workspace")))
+        (pl->ws_bprop && (rc = check_ptr16(workspace, "workspace"))))
         return rc;
     hipStream_t st = (hipStream_t)stream;
     if (pl->dtype == NG_F16) return run_bprop<_Float16>(*pl, F, E, gradI, alpha, workspace, workspace_bytes, st);

@@ -132,9 +132,14 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
     if (!rc) rc = upload(mflat.data(), mflat.size() * sizeof(TapEntry), (void**)&pl->d_merged_flat);
     if (rc) { ng_conv_plan_destroy(pl); return rc; }
 
-    pl->ws_bprop = align_up((size_t)pl->RST * pl->Kpad * pl->Cpad * dtype_size(dtype), 256);
+    // data gradient scratch: the merged filter, or the re-laid filter of the
+    // row-by-row form; the blocked form reads the filter in place
     if (pl->merged)
-        pl->ws_bprop = std::max(pl->ws_bprop, align_up((size_t)pl->m_taps * p.K * pl->m_rpad * dtype_size(dtype), 256));
+        pl->ws_bprop = align_up((size_t)pl->m_taps * p.K * pl->m_rpad * dtype_size(dtype), 256);
+    else if (!pl->bprop_blocked)
+        pl->ws_bprop = align_up((size_t)pl->RST * pl->Kpad * pl->Cpad * dtype_size(dtype), 256);
+    else
+        pl->ws_bprop = 0;
     {
         const int kt = cdiv(p.M * p.P * p.Q * p.N, pl->bk);
         // the most slices any tile shape of the update dispatcher would ask for
