@@ -137,9 +137,20 @@ struct CoreShape {
     int m, n;          // output extents (rows of A-operand, rows of B-operand)
     int k_tiles;       // BK-sized contraction tiles per pass
     int passes;        // contraction passes accumulated into one output (batch_loops)
-    int splits;        // the (passes * k_tiles) tile range is cut into this many slices (gridDim.y)
+    int splits;        // the (passes * k_tiles) tile range is cut into this many slices
     int tiles_m, tiles_n;
 };
+
+// gridDim.y of a launch over `tiles` output tiles (gridDim.x) and `splits`
+// slices: with more than one slice the (tile, slice) pairs are dealt to the XCDs
+// in eight equal contiguous shares (see block_work), which needs 8 * ceil(pairs / 8)
+// workgroups
+inline unsigned grid_slices(int tiles, int splits)
+{
+    if (splits <= 1) return 1u;
+    const long per = ((long)tiles * splits + 7) / 8;
+    return (unsigned)((8 * per + tiles - 1) / tiles);
+}
 
 // Global operand chunks are fetched with raw buffer loads: an offset at or
 // beyond the 2 GiB range of the descriptor returns zeros in hardware, which is
@@ -241,11 +252,8 @@ struct DenseLoader {
 // and numbering the tiles in bands of 8 rows (column-major inside a band) makes
 // such a range a compact block of the output (e.g. 8 x 4 tiles for 32 CUs
 // instead of 16 x 2), so fewer distinct operand tiles pass through its L2.
-__device__ __forceinline__ void tile_of_block(const CoreShape& s, int& tm, int& tn)
+__device__ __forceinline__ void tile_of_block(const CoreShape& s, int pid, int& tm, int& tn)
 {
-    int pid = blockIdx.x;
-    const int total = gridDim.x;
-    if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
     constexpr int BAND = 8;
     const int per_band = BAND * s.tiles_n;
     const int band = pid / per_band;
@@ -254,6 +262,37 @@ __device__ __forceinline__ void tile_of_block(const CoreShape& s, int& tm, int& 
     const int in_band = pid - band * per_band;
     tn = in_band / rows;
     tm = first_m + (in_band - tn * rows);
+}
+
+// Output tile and contraction slice of this workgroup; false: nothing to do.
+// Workgroups are dealt to the 8 XCDs round robin in dispatch order (x fastest,
+// then y).  One slice: an XCD gets a contiguous range of tile numbers (when the
+// tile count is a multiple of 8).  Several slices: the workgroups of one slice
+// read the same contraction range of both operands, so the (slice, tile) pairs,
+// numbered slice-major, are cut into eight equal contiguous shares, one per
+// XCD: an XCD then works on one or two slices at a time and its L2 fetches
+// their operand ranges once, instead of every XCD fetching every slice
+// (measured on a weight gradient: 3.3 GB from HBM where 0.8 GB are needed).
+// gridDim.y is grid_slices().
+__device__ __forceinline__ bool block_work(const CoreShape& s, int& tm, int& tn, int& split)
+{
+    int pid = blockIdx.x;
+    const int total = gridDim.x;
+    if (s.splits > 1) {
+        const unsigned linear = blockIdx.x + gridDim.x * blockIdx.y;
+        const unsigned xcd = linear & 7u, slot = linear >> 3;
+        const unsigned pairs = (unsigned)total * (unsigned)s.splits;
+        const unsigned per = (pairs + 7u) >> 3;
+        const unsigned pair = xcd * per + slot;
+        if (slot >= per || pair >= pairs) return false;
+        split = (int)(pair / (unsigned)total);
+        pid = (int)(pair - (unsigned)split * (unsigned)total);
+    } else {
+        split = 0;
+        if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
+    }
+    tile_of_block(s, pid, tm, tn);
+    return true;
 }
 
 // Scheduling directive for one k-step.  After each MFMA: two LDS reads of the
@@ -345,11 +384,10 @@ void mfma_gemm_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     const int wave = tid >> 6;
     const int wm = wave % WM, wn = wave / WM;
 
-    int tm, tn;
-    tile_of_block(s, tm, tn);
+    int tm, tn, split;
+    if (!block_work(s, tm, tn, split)) return;
     const int m0 = tm * BM, n0 = tn * BN;
     const int z = blockIdx.z;
-    const int split = blockIdx.y;
 
     // contraction tile range of this split
     const int total_tiles = s.passes * s.k_tiles;
@@ -647,11 +685,10 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WM, wn = wave / WM;
 
-    int tm, tn;
-    tile_of_block(s, tm, tn);
+    int tm, tn, split;
+    if (!block_work(s, tm, tn, split)) return;
     const int m0 = tm * BM, n0 = tn * BN;
     const int z = blockIdx.z;
-    const int split = blockIdx.y;
 
     const int total_tiles = s.passes * s.k_tiles;
     const int per = (total_tiles + s.splits - 1) / s.splits;
