@@ -115,7 +115,7 @@ inline int launch_core(const AL& al, const BL& bl, const Epi& epi, int rows, int
     s.passes = 1; s.splits = splits;
     s.tiles_m = cdiv(rows, BM);
     s.tiles_n = cdiv(ncols, BN);
-    launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB>(dim3(s.tiles_m * s.tiles_n, grid_slices(s.tiles_m * s.tiles_n, splits), 1), stream, al, bl, epi, s);
+    launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB>(dim3(grid_tiles(s.tiles_m * s.tiles_n, splits), grid_slices(s.tiles_m * s.tiles_n, splits), 1), stream, al, bl, epi, s);
     NG_CHECK_LAUNCH(what);
     return 0;
 }

@@ -59,7 +59,7 @@ static int launch_gemm(const GemmArgs& g, unsigned sr_bits)
                               (g.flags & NG_FLAG_RELU) ? 1u : 0u, sr_bits, g.seed, g.rng_stream,
                               (((uintptr_t)g.C & 15) == 0 && g.ldc % 8 == 0 && g.ldcz % 8 == 0 && g.n % 8 == 0) ? 1u : 0u};
 
-    dim3 grid(s.tiles_m * s.tiles_n, grid_slices(s.tiles_m * s.tiles_n, s.splits), zcount);
+    dim3 grid(grid_tiles(s.tiles_m * s.tiles_n, s.splits), grid_slices(s.tiles_m * s.tiles_n, s.splits), zcount);
     if (s.splits == 1) {
         launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB, NSTAGE>(grid, g.stream, al, bl, epi, s);
         NG_CHECK_LAUNCH("gemm kernel");

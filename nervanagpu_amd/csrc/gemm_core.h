@@ -145,6 +145,9 @@ struct CoreShape {
 // slices: with more than one slice the (tile, slice) pairs are dealt to the XCDs
 // in eight equal contiguous shares (see block_work), which needs 8 * ceil(pairs / 8)
 // workgroups
+// gridDim.x: the output tiles; a launch with one slice rounds them up to a
+// multiple of 8 so that every XCD can be given one contiguous share
+inline unsigned grid_tiles(int tiles, int splits) { return splits > 1 ? (unsigned)tiles : (unsigned)((tiles + 7) / 8 * 8); }
 inline unsigned grid_slices(int tiles, int splits)
 {
     if (splits <= 1) return 1u;
@@ -266,8 +269,8 @@ __device__ __forceinline__ void tile_of_block(const CoreShape& s, int pid, int& 
 
 // Output tile and contraction slice of this workgroup; false: nothing to do.
 // Workgroups are dealt to the 8 XCDs round robin in dispatch order (x fastest,
-// then y).  One slice: an XCD gets a contiguous range of tile numbers (when the
-// tile count is a multiple of 8).  Several slices: the workgroups of one slice
+// then y).  One slice: an XCD gets a contiguous eighth of the tile numbers
+// (gridDim.x is grid_tiles(); surplus workgroups leave).  Several slices: the workgroups of one slice
 // read the same contraction range of both operands, so the (slice, tile) pairs,
 // numbered slice-major, are cut into eight equal contiguous shares, one per
 // XCD: an XCD then works on one or two slices at a time and its L2 fetches
@@ -276,8 +279,8 @@ __device__ __forceinline__ void tile_of_block(const CoreShape& s, int pid, int& 
 // gridDim.y is grid_slices().
 __device__ __forceinline__ bool block_work(const CoreShape& s, int& tm, int& tn, int& split)
 {
-    int pid = blockIdx.x;
-    const int total = gridDim.x;
+    int pid;
+    const int total = s.tiles_m * s.tiles_n;
     if (s.splits > 1) {
         const unsigned linear = blockIdx.x + gridDim.x * blockIdx.y;
         const unsigned xcd = linear & 7u, slot = linear >> 3;
@@ -289,7 +292,10 @@ __device__ __forceinline__ bool block_work(const CoreShape& s, int& tm, int& tn,
         pid = (int)(pair - (unsigned)split * (unsigned)total);
     } else {
         split = 0;
-        if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
+        const int per = (total + 7) >> 3;
+        const int slot = (int)(blockIdx.x >> 3);
+        pid = (int)(blockIdx.x & 7u) * per + slot;
+        if (pid >= total) return false;
     }
     tile_of_block(s, pid, tm, tn);
     return true;
