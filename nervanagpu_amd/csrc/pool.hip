@@ -95,7 +95,7 @@ struct PoolGeom {
     // backward by cells (pool_bprop_cell_kernel): which compiled (window, stride)
     // shape applies (0: none) and the number of stride-sized cells along h and w
     // that hold at least one input element
-    int use_cells, cells_h, cells_w;
+    int use_cells, cells_h, cells_w, cell_remap;
     FastDiv div_ch, div_cw;
 };
 
@@ -415,7 +415,7 @@ void pool_bprop_cell_kernel(const T* __restrict__ E, const unsigned char* __rest
     constexpr int NW = (RS + STR - 1) / STR;
     typedef typename Pack<T, VEC>::raw_t raw_t;
     const unsigned per_map = (unsigned)(g.D * g.cells_h * g.cells_w * g.nvec);
-    const unsigned inner = blockIdx.x * 256u + threadIdx.x;
+    const unsigned inner = xcd_block_index(g.cell_remap) * 256u + threadIdx.x;
     int nv, cx, cy, z;
     if (!split_inner(inner, per_map, g.div_nvec, g.div_cw, g.div_ch, g.nvec, g.cells_w, g.cells_h, nv, cx, cy, z)) return;
     // one feature map holds fewer than 2^31 elements: 32-bit offsets inside it
@@ -587,6 +587,10 @@ static PoolGeom make_geom(const ng_pool_params& p, int vec, size_t elem_bytes)
     g.use_cells = 0;
     g.cells_h = (p.H - 1 + p.pad_h) / p.str_h + 1;
     g.cells_w = (p.W - 1 + p.pad_w) / p.str_w + 1;
+    // neighbouring cells read the same windows: XCD-contiguous numbering as in the
+    // forward kernels, for overlapping windows and maps of 64 workgroups or more
+    // (rounding a smaller grid up to a multiple of 8 idles too many of them)
+    g.cell_remap = (!disjoint && (long)p.D * g.cells_h * g.cells_w * g.nvec >= 64 * 256) ? 1 : 0;
     g.div_ch = FastDiv::make((unsigned)g.cells_h);
     g.div_cw = FastDiv::make((unsigned)g.cells_w);
     return g;
@@ -673,7 +677,7 @@ static void launch_gather(const PoolGeom& g, bool win2, dim3 grid, const T* E, c
                           hipStream_t st)
 {
     if constexpr (VEC > 1) {
-        const dim3 cgrid = grid_for((long)g.D * g.cells_h * g.cells_w * g.nvec, g.C);
+        const dim3 cgrid = grid_for((long)g.D * g.cells_h * g.cells_w * g.nvec, g.C, g.cell_remap);
         switch (g.use_cells) {
         case 0x32:
             hipLaunchKernelGGL((pool_bprop_cell_kernel<T, VEC, OP, 3, 2>), cgrid, dim3(256), 0, st, E, arg, B, g);
