@@ -16,16 +16,16 @@ static int fprop_tile(const ConvPlan& pl, const void* I, const void* F, void* O,
     const PixelLattice lat = PixelLattice::make(p.N, ncols, p.Q, p.P * p.Q);
     if (BLOCKED) {
         const int nblk = cdiv(p.C, BK);
-        FilterBlockLoader<T, BK> al{(const T*)F, p.K, pl.RST * p.K, FastDiv::make((unsigned)nblk), nblk, p.C};
+        FilterBlockLoader<T, BK> al{(const T*)F, p.K, pl.RST * p.K, FastDiv::make((unsigned)pl.RST), pl.RST, p.C};
         GatherColsLoader<T, TIN, true, BK> bl{(const TIN*)I, pl.d_fprop_taps, pl.CRST, lat,
                                               p.str_d, p.str_h, p.str_w, p.D, p.H, p.W,
-                                              DHWN, FastDiv::make((unsigned)nblk), nblk, p.C};
+                                              DHWN, FastDiv::make((unsigned)pl.RST), nblk, p.C, pl.RST};
         return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, epi, p.K, ncols, pl.RST * nblk, 1, stream, "conv fprop");
     } else {
         DenseLoader<T, MC, true> al{(const T*)F, 0, p.K, p.K, pl.CRST};
         GatherColsLoader<T, TIN, false, BK> bl{(const TIN*)I, pl.d_fprop_flat, pl.CRST, lat,
                                                p.str_d, p.str_h, p.str_w, p.D, p.H, p.W,
-                                               0, FastDiv{0, 0}, 1, 0};
+                                               0, FastDiv{0, 0}, 1, 0, 0};
         return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, epi, p.K, ncols, cdiv(pl.CRST, BK), 1, stream, "conv fprop");
     }
 }

@@ -105,6 +105,15 @@ struct PixelLattice {
 
 #define NG_FAR (-0x40000000)
 
+// contraction tile index -> (tap, channel block); div divides by nblk when
+// block_major_taps == 0 and by block_major_taps otherwise
+__device__ __forceinline__ void decode_tile(int kt, const FastDiv& div, int nblk, int block_major_taps, int& tap, int& blk)
+{
+    const int hi = (int)div.div((unsigned)kt);
+    if (block_major_taps) { blk = hi; tap = kt - hi * block_major_taps; }
+    else                  { tap = hi; blk = kt - hi * nblk; }
+}
+
 // B operand of fprop / bprop (row-contiguous tile: lines are contraction rows,
 // columns are (pixel, n)).  Gathered coordinate of a tap at lattice point
 // (iz,iy,ix) is (iz*gs_d + dz, iy*gs_h + dy, ix*gs_w + dx) inside a
@@ -118,9 +127,16 @@ struct GatherColsLoader {
     int             gs_d, gs_h, gs_w;
     int             lim_d, lim_h, lim_w;
     int             row_stride; // BLOCKED: elements between consecutive rows of a block
-    FastDiv         blk_div;    // BLOCKED: tile index -> tap (blocks per tap = nblk)
+    FastDiv         blk_div;    // BLOCKED: tile index / nblk (blocks per tap) or / ntaps, see block_major
     int             nblk;
     int             chan;       // BLOCKED: rows per tap; the last block of a tap may be partly empty
+    // BLOCKED tile order.  0: tap-major (all channel blocks of a tap, then the next
+    // tap).  ntaps > 0: block-major (all taps of a channel block, then the next
+    // block): the taps of one block re-read the same activations shifted by a
+    // pixel or a row, so the share an XCD works on stays in its L2 across the
+    // taps (tap-major re-fetched the data gradient's E of a 5x5 layer 8.7 times
+    // from HBM).  The A operand's loader must use the same order.
+    int             block_major_taps;
 
     // same-type inputs are plain 16-byte buffer loads (see DenseLoader::DIRECT)
     static constexpr bool DIRECT = std::is_same<T, TIN>::value;
@@ -149,8 +165,8 @@ struct GatherColsLoader {
         t.rsrc = make_rsrc(X);
         t.k0 = k0;
         if (BLOCKED) {
-            const int tap = (int)blk_div.div((unsigned)kt);
-            const int blk = kt - tap * nblk;
+            int tap, blk;
+            decode_tile(kt, blk_div, nblk, block_major_taps, tap, blk);
             const TapEntry e = tab[tap];
             t.toff = e.off + blk * BK * row_stride;
             t.dz = e.dz; t.dy = e.dy; t.dx = e.dx;
@@ -193,8 +209,8 @@ struct FilterBlockLoader {
     const T* F;
     int      K;          // row length (output feature maps)
     int      RSTK;       // elements between consecutive channels
-    FastDiv  blk_div;
-    int      nblk;
+    FastDiv  tap_div;    // tile index -> channel block (block-major order, ntaps tiles per block)
+    int      ntaps;
     int      C;          // channels
 
     static constexpr bool DIRECT = true;
@@ -212,8 +228,8 @@ struct FilterBlockLoader {
     }
     __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/) const
     {
-        const int tap = (int)blk_div.div((unsigned)kt);
-        const int blk = kt - tap * nblk;
+        const int blk = (int)tap_div.div((unsigned)kt);
+        const int tap = kt - blk * ntaps;
         Tile t;
         t.rsrc = make_rsrc(F + (long)blk * BK * RSTK + (long)tap * K);
         t.rows = C - blk * BK;
@@ -239,8 +255,8 @@ struct FilterRowsLoader {
     int        C;         // rows
     int        K;         // contraction extent per tap
     int        RSTK;      // elements between consecutive rows
-    FastDiv    blk_div;   // tile index -> tap (blocks per tap = nblk)
-    int        nblk;
+    FastDiv    tap_div;   // tile index -> block of output maps (block-major order, ntaps tiles per block)
+    int        ntaps;
 
     static constexpr bool DIRECT = true;
     static constexpr bool TILE_READS_TABLE = true;
@@ -257,8 +273,8 @@ struct FilterRowsLoader {
     }
     __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/) const
     {
-        const int tap = (int)blk_div.div((unsigned)kt);
-        const int blk = kt - tap * nblk;
+        const int blk = (int)tap_div.div((unsigned)kt);
+        const int tap = kt - blk * ntaps;
         Tile t;
         // the table entry is wavefront-uniform; the descriptor must live in scalar registers
         const int trs = __builtin_amdgcn_readfirstlane(tap_trs[tap]);
