@@ -32,12 +32,7 @@ static int launch_update(const ConvPlan& pl, const void* I, const void* E, void*
     PartialEpilogue pe{(float*)ws, rows, cols, 1, 1u};
     int rc = launch_core<T, BM, BN, BK, WM, WN, KC, KC>(al, bl, pe, rows, cols, k_tiles, splits, stream, "conv update");
     if (rc) return rc;
-    const long total = (long)rows * cols;
-    const unsigned vec8 = (cols % 8 == 0) ? 1u : 0u;
-    const long items = vec8 ? total / 8 : total;
-    const int blocks = (int)std::min<long>((items + 255) / 256, 16384);
-    hipLaunchKernelGGL((splitk_reduce_kernel<TOUT, ScaleStoreEpilogue<TOUT>>), dim3(blocks), dim3(256), 0,
-                       stream, (const float*)ws, splits, 1, rows, cols, epi, vec8);
+    launch_splitk_reduce<TOUT, ScaleStoreEpilogue<TOUT>>((const float*)ws, splits, 1, rows, cols, epi, stream);
     NG_CHECK_LAUNCH("conv update reduce");
     return 0;
 }

@@ -67,12 +67,7 @@ static int launch_gemm(const GemmArgs& g, unsigned sr_bits)
         PartialEpilogue pe{(float*)g.ws, g.m, g.n, zcount, (g.n % 8 == 0) ? 1u : 0u};
         launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB, NSTAGE>(grid, g.stream, al, bl, pe, s);
         NG_CHECK_LAUNCH("gemm split kernel");
-        const long total = (long)zcount * g.m * g.n;
-        const unsigned vec8 = (g.n % 8 == 0) ? 1u : 0u;
-        const long items = vec8 ? total / 8 : total;
-        const int blocks = (int)std::min<long>((items + 255) / 256, 16384);
-        hipLaunchKernelGGL((splitk_reduce_kernel<T, ScaleStoreEpilogue<T>>), dim3(blocks), dim3(256), 0, g.stream,
-                           (const float*)g.ws, s.splits, zcount, g.m, g.n, epi, vec8);
+        launch_splitk_reduce<T, ScaleStoreEpilogue<T>>((const float*)g.ws, s.splits, zcount, g.m, g.n, epi, g.stream);
         NG_CHECK_LAUNCH("gemm split reduce");
     }
     return 0;

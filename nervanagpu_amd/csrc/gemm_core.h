@@ -1066,6 +1066,79 @@ void splitk_reduce_kernel(const float* __restrict__ ws, int splits, int zcount, 
     }
 }
 
+// The same reduction for outputs too small to fill the chip with one thread
+// per 8 columns (weight gradients of small filters cut into a hundred or more
+// slices): 2^lanes_log2 lanes share a group of 8 columns, lane l adds slices
+// l, l + L, ... in order, and an exchange tree over the lanes of the group adds
+// the lane sums.  The order of the additions depends only on (splits, L), so
+// results are reproducible.  n must be a multiple of 8.
+template <typename T, class Epi>
+__global__ __launch_bounds__(256)
+void splitk_reduce_lanes_kernel(const float* __restrict__ ws, int splits, int zcount, int m, int n, Epi epi,
+                                int lanes_log2)
+{
+    const long total = (long)zcount * m * n;
+    const long groups = total >> 3;
+    const int per_row = n >> 3;
+    const int L = 1 << lanes_log2;
+    const int gpw = 64 >> lanes_log2;            // groups per wavefront
+    const int lane = threadIdx.x & 63;
+    const int gi = lane & (gpw - 1);             // consecutive lanes read consecutive groups
+    const int l = lane >> (6 - lanes_log2);
+    const long wave = ((long)blockIdx.x * 256 + threadIdx.x) >> 6;
+    const long nwaves = (long)gridDim.x * 4;
+    for (long gb = wave * gpw; gb < groups; gb += nwaves * gpw) {
+        const long g = gb + gi;
+        float acc[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] = 0.0f;
+        if (g < groups) {
+            const float* p = ws + g * 8;
+#pragma unroll 2
+            for (int sidx = l; sidx < splits; sidx += L) {
+                const float4_t lo = *reinterpret_cast<const float4_t*>(p + sidx * total);
+                const float4_t hi = *reinterpret_cast<const float4_t*>(p + sidx * total + 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) { acc[e] += lo[e]; acc[e + 4] += hi[e]; }
+            }
+        }
+        for (int mask = gpw; mask < 64; mask <<= 1) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[e] += __shfl_xor(acc[e], mask, 64);
+        }
+        if (l == 0 && g < groups) {
+            const long r = g / per_row;
+            const int j0 = (int)(g - r * per_row) * 8;
+            epi.store8((int)(r % m), j0, (int)(r / m), 0, acc);
+        }
+    }
+}
+
+// sum the `splits` partial slices in the scratch arena and run the epilogue
+template <typename T, class Epi>
+inline void launch_splitk_reduce(const float* ws, int splits, int zcount, int m, int n, const Epi& epi,
+                                 hipStream_t stream)
+{
+    const long total = (long)zcount * m * n;
+    const unsigned vec8 = (n % 8 == 0) ? 1u : 0u;
+    const long items = vec8 ? total / 8 : total;
+    // lanes per group: until the launch has about two wavefronts per SIMD, every
+    // lane keeping at least two slices
+    int lanes_log2 = 0;
+    const long want = (long)device_cu_count() * 512;
+    while (vec8 && lanes_log2 < 6 && (items << (lanes_log2 + 1)) <= want && (4 << lanes_log2) <= splits) lanes_log2++;
+    if (lanes_log2 > 0) {
+        const long threads = items << lanes_log2;
+        const int blocks = (int)std::min<long>((threads + 255) / 256, 16384);
+        hipLaunchKernelGGL((splitk_reduce_lanes_kernel<T, Epi>), dim3(blocks), dim3(256), 0, stream,
+                           ws, splits, zcount, m, n, epi, lanes_log2);
+    } else {
+        const int blocks = (int)std::min<long>((items + 255) / 256, 16384);
+        hipLaunchKernelGGL((splitk_reduce_kernel<T, Epi>), dim3(blocks), dim3(256), 0, stream,
+                           ws, splits, zcount, m, n, epi, vec8);
+    }
+}
+
 // Launch the contraction core: the direct-to-LDS pipeline when both operands
 // are plain 16-byte buffer loads of 16-bit elements, the register-staged one
 // otherwise (fp32, element-wise edge handling, 8-bit inputs converted on load).

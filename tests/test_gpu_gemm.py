@@ -73,6 +73,28 @@ def test_dot_aligned_ragged_edges(ng, dtype, op):
                acc_atol(_absdot(A, B)))
 
 
+# small outputs over long contractions: the contraction is cut into many slices
+# and the fp32 partial sums are added by several lanes per output group
+LONG_K = [(64, 64, 8192), (72, 136, 16400), (200, 8, 32768), (8, 24, 4104)]
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("op", ["nn", "nt", "tn"])
+def test_dot_long_contraction_small_output(ng, dtype, op):
+    rng = np.random.default_rng(17)
+    for (m, n, k) in LONG_K:
+        A, B, dA, dB = _operands(ng, op, m, n, k, dtype, rng)
+        C = ng.empty((m, n), dtype=dtype)
+        ng.dot(dA, dB, C, relu=True)
+        first = C.get()
+        _check(first, orc.ref_dot(A, B, relu=True), dtype, "%s %s m,n,k=%d,%d,%d" % (np.dtype(dtype), op, m, n, k),
+               acc_atol(_absdot(A, B)))
+        # the order of the additions is fixed: a second run gives the same bits
+        C.fill(0)
+        ng.dot(dA, dB, C, relu=True)
+        assert np.array_equal(first.view(np.uint8), C.get().view(np.uint8))
+
+
 @pytest.mark.parametrize("op", ["nn", "tn"])
 def test_config1_fp32_1024(ng, op):
     rng = np.random.default_rng(0)
