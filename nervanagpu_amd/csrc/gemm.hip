@@ -104,10 +104,12 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
     if (!operands_vectorizable<_Float16>(g)) return launch_layout<_Float16, 128, 128, 64, 2, 2, false>(g, sr_bits);
     const int cus = device_cu_count();
     const int k_tiles = ceil_div(g.k, 64) * g.batch_loops;
-    // 256x256 tiles when they still fill the chip and the contraction is long
-    // enough to amortise their prologue and epilogue
+    // 256x256 tiles when they cover more than half the chip and the contraction
+    // is long enough to amortise their prologue and epilogue (exactly half the
+    // chip is one full round of 128x128 tiles at two workgroups per CU, which is
+    // a third faster)
     const long big_tiles = (long)ceil_div(g.m, 256) * ceil_div(g.n, 256) * g.batch_grid;
-    if (g.m >= 256 && g.n >= 256 && big_tiles >= cus / 2 && k_tiles >= 8)
+    if (g.m >= 256 && g.n >= 256 && big_tiles > cus / 2 && k_tiles >= 8)
         return launch_layout<_Float16, 256, 256, 64, 2, 4, true>(g, sr_bits);
     // minibatch-wide outputs (n <= 128) stream the weight matrix: halve the row
     // tile so that fewer contraction slices, i.e. fewer fp32 partials, fill the chip
