@@ -59,11 +59,14 @@ inline bool blocks_pay(int channels, int bk) { return channels % bk == 0 || 2 * 
 // second workgroup on half of the CUs overlaps the tile-step latency of the
 // first), one per CU for short contractions, where the extra fp32 partials
 // cost more than the overlap gains
-inline int conv_splits(int out_tiles, int total_k_tiles, size_t slice_bytes, size_t ws_bytes)
+// (`halves`: workgroups per CU in halves; the 64x64 tile of the smallest
+// filters needs a fifth of the LDS and gains from three per CU: VGG conv1
+// weight gradient 119 -> 86 us)
+inline int conv_splits(int out_tiles, int total_k_tiles, size_t slice_bytes, size_t ws_bytes, int halves = 3)
 {
     const int cus = device_cu_count();
     if (out_tiles >= cus || total_k_tiles < 8) return 1;
-    int splits = cdiv(3 * cus / 2, out_tiles);
+    int splits = cdiv(halves * cus / 2, out_tiles);
     if (total_k_tiles / splits < 30) splits = cdiv(cus, out_tiles);
     splits = std::min(splits, total_k_tiles / 4);
     if (slice_bytes) splits = (int)std::min<size_t>((size_t)splits, ws_bytes / slice_bytes);

@@ -143,8 +143,9 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
     {
         const int kt = cdiv(p.M * p.P * p.Q * p.N, pl->bk);
         // the most slices any tile shape of the update dispatcher would ask for
-        const int splits = std::max(conv_splits(cdiv(pl->CRST, 128) * cdiv(p.K, 128), kt, 0, 0),
-                                    conv_splits(cdiv(pl->CRST, 256) * cdiv(p.K, 256), kt, 0, 0));
+        int splits = std::max(conv_splits(cdiv(pl->CRST, 128) * cdiv(p.K, 128), kt, 0, 0),
+                              conv_splits(cdiv(pl->CRST, 256) * cdiv(p.K, 256), kt, 0, 0));
+        if (p.K <= 64 && pl->CRST <= 64) splits = std::max(splits, conv_splits(1, kt, 0, 0, 6));
         pl->ws_update = splits > 1 ? align_up((size_t)splits * pl->CRST * p.K * sizeof(float), 256) : 0;
     }
     *plan_out = pl;

@@ -17,7 +17,7 @@ static int launch_update(const ConvPlan& pl, const void* I, const void* E, void*
     const int k_tiles = cdiv(kdim, BK);
     const int tiles = cdiv(rows, BM) * cdiv(cols, BN);
     const size_t slice = (size_t)rows * cols * sizeof(float);
-    const int splits = ws ? conv_splits(tiles, k_tiles, slice, ws_bytes) : 1;
+    const int splits = ws ? conv_splits(tiles, k_tiles, slice, ws_bytes, (BM == 64 && BN == 64) ? 6 : 3) : 1;
     const int npt = BLOCKED ? p.N / BK : 1;
 
     GatherRowsLoader<T, TIN, BLOCKED, BK> al{(const TIN*)I, pl.d_fprop_flat, pl.CRST, p.N, kdim, p.Q, p.P * p.Q,
