@@ -73,6 +73,18 @@ def test_dot_aligned_ragged_edges(ng, dtype, op):
                acc_atol(_absdot(A, B)))
 
 
+@pytest.mark.parametrize("op", ["nn", "nt", "tn"])
+def test_dot_mid_size_long_contraction_fp16(ng, op):
+    # between half a chip and a chip of 128x128 tiles with 48 or more 64-deep
+    # contraction tiles: 128x128 tiles in two slices, ragged in m, n and k
+    rng = np.random.default_rng(19)
+    m, n, k = 1544, 1800, 3080
+    A, B, dA, dB = _operands(ng, op, m, n, k, np.float16, rng)
+    C = ng.empty((m, n), dtype=np.float16)
+    ng.dot(dA, dB, C)
+    _check(C.get(), orc.ref_dot(A, B), np.float16, "float16 %s m,n,k=%d,%d,%d" % (op, m, n, k), acc_atol(_absdot(A, B)))
+
+
 # small outputs over long contractions: the contraction is cut into many slices
 # and the fp32 partial sums are added by several lanes per output group
 LONG_K = [(64, 64, 8192), (72, 136, 16400), (200, 8, 32768), (8, 24, 4104)]
