@@ -973,6 +973,22 @@ struct ScaleStoreEpilogue {
 #pragma unroll
             for (int q = 0; q < NV; q++)
                 reinterpret_cast<uint4_t*>(p)[q] = reinterpret_cast<const uint4_t*>(out)[q];
+        } else if (vec && sizeof(bits_t) == 2 && sr_bits == 10u) {
+            // fp16 at the full 10 bits: pairs share a draw and a packed convert
+            bits_t cur[8];
+            if (beta != 0.0f) *reinterpret_cast<uint4_t*>(cur) = *reinterpret_cast<const uint4_t*>(p);
+            const unsigned pair0 = rng_index(i, j0, z) >> 1;
+            unsigned packed[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                float v0 = scale(acc[2 * q]), v1 = scale(acc[2 * q + 1]);
+                if (beta != 0.0f) {
+                    v0 += beta * StoreBits<T>::widen(cur[2 * q]);
+                    v1 += beta * StoreBits<T>::widen(cur[2 * q + 1]);
+                }
+                packed[q] = ng_sr10_f16x2(v0, v1, ng_rand32(seed, stream, pair0 + q));
+            }
+            *reinterpret_cast<uint4_t*>(p) = *reinterpret_cast<const uint4_t*>(packed);
         } else if (vec) {
             bits_t out[8];
             if (beta != 0.0f) {

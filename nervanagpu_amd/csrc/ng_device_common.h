@@ -91,6 +91,30 @@ NG_DEV unsigned short ng_sr_f16(float v, unsigned bits, unsigned r)
     return ng_f32_to_f16_rz(__uint_as_float((u & 0x80000000u) | m2));
 }
 
+// The same rounding when all 10 mantissa bits of fp16 are kept, in fewer
+// operations.  The truncating convert drops exactly the bits the mask would
+// clear; bounding the sum by max(mag, largest finite fp32) keeps the increment
+// from carrying a finite value into the infinity pattern (the convert then
+// saturates at 65504 as the clamp did) and leaves infinities and NaNs as they
+// are.  Returns the fp32 value whose truncating convert is the result.
+NG_DEV float ng_sr10_bump(float v, unsigned r13)
+{
+    const unsigned u   = __float_as_uint(v);
+    const unsigned mag = u & 0x7FFFFFFFu;
+    const unsigned m2  = min(mag + r13, max(mag, 0x7F7FFFFFu));
+    return __uint_as_float((u & 0x80000000u) | m2);
+}
+
+// Two neighbouring elements sharing the draw h (even element: its high half,
+// odd element: its low half, as in ng_rand_sr16) -> packed pair of fp16 bits.
+NG_DEV unsigned ng_sr10_f16x2(float v_even, float v_odd, unsigned h)
+{
+    typedef _Float16 ng_half2_t __attribute__((ext_vector_type(2)));
+    const ng_half2_t p = __builtin_bit_cast(
+        ng_half2_t, __builtin_amdgcn_cvt_pkrtz(ng_sr10_bump(v_even, h >> 19), ng_sr10_bump(v_odd, (h >> 3) & 0x1FFFu)));
+    return __builtin_bit_cast(unsigned, p);
+}
+
 // nearest-even fp32 -> fp16 bits
 NG_DEV unsigned short ng_f32_to_f16_rn(float v)
 {

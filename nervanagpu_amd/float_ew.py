@@ -392,6 +392,25 @@ def generate_source(spec, name="ew_kernel"):
             o.append("%sconst unsigned rh%d_ = ng_rand32(rng_seed, rng_stream, (rng_idx >> 1) + %du);" % (pad, k, k))
         return ["rh%d_" % (v // 2) if v % 2 == 0 else "(rh%d_ << 16)" % (v // 2) for v in range(V)]
 
+    def rounded_vector(o, pad, code, vals, rwords, idx_of):
+        """statements that fill the vector o_ with the rounded values"""
+        paired = rwords[0] is not None and V % 2 == 0
+        if paired:
+            # all 10 mantissa bits kept: pairs share a draw and a packed convert
+            o.append("%sif (sr_bits == 10u) {" % pad)
+            if V == 2:
+                o.append("%s  o_ = __builtin_bit_cast(vt_, ng_sr10_f16x2(%s, %s, rh0_));" % (pad, vals[0], vals[1]))
+            else:
+                o.append("%s  typedef unsigned qt_ __attribute__((ext_vector_type(%d))); qt_ q_;" % (pad, V // 2))
+                for k in range(V // 2):
+                    o.append("%s  q_[%d] = ng_sr10_f16x2(%s, %s, rh%d_);" % (pad, k, vals[2 * k], vals[2 * k + 1], k))
+                o.append("%s  o_ = __builtin_bit_cast(vt_, q_);" % pad)
+            o.append("%s} else {" % pad)
+        for v in range(V):
+            o.append("%so_[%d] = %s;" % (pad, v, _gen_round(code, vals[v], rounding, idx_of(v), rwords[v])))
+        if paired:
+            o.append("%s}" % pad)
+
     def store_code(item, base_col, vals, indent):
         pad = " " * indent
         arg_id, code, access, take_axis, _ = out_t
@@ -400,8 +419,8 @@ def generate_source(spec, name="ew_kernel"):
         if access == "vec" and V > 1:
             o.append("%s{ typedef %s vt_ __attribute__((ext_vector_type(%d))); vt_ o_;" % (pad, ct, V))
             rwords = pair_words(o, pad + "  ", code)
-            for v in range(V):
-                o.append("%s  o_[%d] = %s;" % (pad, v, _gen_round(code, vals[v], rounding, "rng_idx + %du" % v if not rng_strided else "rng_idx + %du * rng_cm" % v, rwords[v])))
+            rounded_vector(o, pad + "  ", code, vals, rwords,
+                           lambda v: "rng_idx + %du" % v if not rng_strided else "rng_idx + %du * rng_cm" % v)
             o.append("%s  *reinterpret_cast<vt_*>(p%d + (long)(%s)) = o_; }" % (pad, arg_id, base_col))
         else:
             for v in range(V):
@@ -451,8 +470,7 @@ def generate_source(spec, name="ew_kernel"):
         if V > 1:
             L.append("        { typedef %s vt_ __attribute__((ext_vector_type(%d))); vt_ o_;" % (ct, V))
             rwords = pair_words(L, "          ", code)
-            for v in range(V):
-                L.append("          o_[%d] = %s;" % (v, _gen_round(code, vals[v], rounding, "rng_idx + %du" % v, rwords[v])))
+            rounded_vector(L, "          ", code, vals, rwords, lambda v: "rng_idx + %du" % v)
             L.append("          *reinterpret_cast<vt_*>(p%d + col) = o_; }" % arg_id)
         else:
             L.append("        p%d[col] = %s;" % (arg_id, _gen_round(code, vals[0], rounding, "rng_idx")))

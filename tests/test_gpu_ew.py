@@ -315,12 +315,23 @@ def test_stochastic_rounding_store_bit_exact(ng):
     r = orc.rand32(77, ngs.rng_counter, np.arange(a.size, dtype=np.uint32)).reshape(a.shape)
     assert np.array_equal(F.get().view(np.uint32), orc.round_stochastic_fp32(a, 15, r).view(np.uint32))
     # special values through the device conversion
-    sp = np.array([[0.0, -0.0, 65504.0, 65519.0, 70000.0, -70000.0, 1e-8, 6e-8, 6.1e-5, -3e-5, 1e30, 2.0 ** -24]],
-                  dtype=np.float32)
+    sp = np.array([0.0, -0.0, 65504.0, 65519.0, 70000.0, -70000.0, 1e-8, 6e-8, 6.1e-5, -3e-5, 1e30, 2.0 ** -24,
+                   np.inf, -np.inf, 3.4028235e38, -3.4028235e38, 3.4028e38, 65503.99, 65535.99, 65536.0,
+                   2.0 ** -14, 2.0 ** -14 - 2.0 ** -30, 5.9e-8, -2.9e-8], dtype=np.float32)
+    spb = np.concatenate([sp.view(np.uint32), np.array([0x7FC00000, 0xFFC00000, 0x7F800001, 0xFFFFFFFF, 0x7FFFFFFF,
+                                                        0x7F7FE000, 0x7F7FE001, 0x477FDFFF], dtype=np.uint32)])
+    # every value at even and odd positions, under many different draws, at full and reduced precision
+    sp = np.tile(spb, 64).reshape(64, spb.size).view(np.float32)
+    sp = np.concatenate([sp, np.roll(sp, 1, axis=1)], axis=0)
     S = ngs.empty(sp.shape)
-    S[:] = ngs.array(sp, dtype=np.float32)
-    r = orc.rand_sr16(77, ngs.rng_counter, np.arange(sp.size, dtype=np.uint32)).reshape(sp.shape)
-    assert np.array_equal(S.get().view(np.uint16), orc.round_stochastic_fp16(sp, 10, r).view(np.uint16))
+    for bits in (10, 7):
+        S.rounding = bits
+        S[:] = ngs.array(sp, dtype=np.float32)
+        r = orc.rand_sr16(77, ngs.rng_counter, np.arange(sp.size, dtype=np.uint32)).reshape(sp.shape)
+        got, ref = S.get().view(np.uint16), orc.round_stochastic_fp16(sp, bits, r).view(np.uint16)
+        nan = np.isnan(sp)
+        assert np.array_equal(got[~nan], ref[~nan]), bits
+        assert np.all(np.isnan(S.get()[nan]))   # NaN stays NaN (payload bits are not compared)
 
 
 def ng_mean0(ngs, A):
