@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 
 import oracle as orc
+from oracle import ref_numpy as rn
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 
@@ -138,3 +139,38 @@ def test_fast_ew_dims():
     assert orc.fast_ew_dims(96)[0] == (1, 96)
     shp, strd = orc.fast_ew_dims(7 * 13)
     assert shp[0] * shp[1] == 91 and strd == (shp[1], 1)
+
+
+def test_sr10_short_form_is_the_same_function():
+    """The device rounds at the default 10 bits with a shorter expression
+    (ng_sr10_bump in csrc/ng_device_common.h): no mask, and the sum bounded by
+    max(magnitude, largest finite fp32) instead of clamp + infinity test.  It
+    must be the oracle's function bit for bit, NaN payloads included."""
+    U = np.uint32
+
+    def short_form(x, r):
+        u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+        mag = u & U(0x7FFFFFFF)
+        with np.errstate(over="ignore"):
+            t = np.minimum(mag + (r >> U(19)), np.maximum(mag, U(0x7F7FFFFF)))
+        return rn.f32_to_f16_rz(((u & U(0x80000000)) | t).astype(np.uint32).view(np.float32))
+
+    rng = np.random.default_rng(3)
+    for case in range(4):
+        bits = rng.integers(0, 2 ** 32, 500_000, dtype=np.uint64).astype(np.uint32)
+        if case == 1:    # exponents around the fp16 range, subnormal results included
+            bits = (bits & U(0x807FFFFF)) | (rng.integers(100, 146, bits.size).astype(np.uint32) << U(23))
+        if case == 2:    # around the largest finite fp32, infinities and NaNs
+            bits = (bits & U(0x8000FFFF)) | U(0x7F7F0000) | ((bits >> U(3)) & U(0x00810000))
+        r = rng.integers(0, 2 ** 32, bits.size, dtype=np.uint64).astype(np.uint32)
+        if case == 3:
+            r |= U(0xFFF80000)
+        ref = orc.round_stochastic_fp16(bits.view(np.float32), 10, r).view(np.uint16)
+        assert np.array_equal(ref, short_form(bits.view(np.float32), r).view(np.uint16))
+    sp = np.array([0x7F800000, 0xFF800000, 0x7FC00000, 0xFFFFFFFF, 0x7FFFFFFF, 0x7F7FFFFF, 0xFF7FFFFF, 0x7F7FE000,
+                   0x7F7FE001, 0x477FE000, 0x477FDFFF, 0x477FFFFF, 0x47800000, 0, 0x80000000, 1, 0x33800000,
+                   0x337FFFFF, 0x38800000, 0x387FFFFF], dtype=np.uint32)
+    for rv in (0, 0xFFFFFFFF, 0x80000000, 0x0007FFFF, 0xFFF80000):
+        r = np.full(sp.shape, rv, dtype=np.uint32)
+        assert np.array_equal(orc.round_stochastic_fp16(sp.view(np.float32), 10, r).view(np.uint16),
+                              short_form(sp.view(np.float32), r).view(np.uint16))
