@@ -6,7 +6,7 @@ Benchmark of the NervanaGPU compute core on one MI355X.
     python bench.py --all [--out FILE]                    -> also a per-case table
                                                              (GEMM, conv, pool, elementwise)
 
-A "step" is one pass over BASELINE config 2: the fp16 fully-connected GEMM sweep
+A "step" is one pass over benchmark configuration 2: the fp16 fully-connected GEMM sweep
 with minibatch 128 ((M,K) in {(4096,9216),(4096,4096),(1000,4096)} x nn/nt/tn x
 relu off/on x nearest/stochastic rounding), the square 4096^3 fp16 GEMM and the
 batched 32 x 512^3 GEMM, with every operand already resident in HBM.  `value` is

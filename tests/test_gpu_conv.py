@@ -124,10 +124,10 @@ def test_conv_adjoint_identity_gpu(ng):
     assert abs(a - b) <= 1e-5 * abs(a) and abs(a - c) <= 1e-5 * abs(a)
 
 
-ALEXNET = [  # C,H,W,K,R,S,stride,pad at N=128 (BASELINE config 3)
+ALEXNET = [  # C,H,W,K,R,S,stride,pad at N=128 (benchmark configuration 3)
     (3, 224, 224, 64, 11, 11, 4, 2), (64, 27, 27, 192, 5, 5, 1, 2), (192, 13, 13, 384, 3, 3, 1, 1),
     (384, 13, 13, 256, 3, 3, 1, 1), (256, 13, 13, 256, 3, 3, 1, 1)]
-VGG = [  # C,HW,K at N=64, 3x3 s1 p1 (BASELINE config 4)
+VGG = [  # C,HW,K at N=64, 3x3 s1 p1 (benchmark configuration 4)
     (3, 224, 64), (64, 224, 64), (64, 112, 128), (128, 112, 128), (128, 56, 256), (256, 56, 256),
     (256, 28, 512), (512, 28, 512), (512, 14, 512)]
 
