@@ -187,8 +187,12 @@ int ng_pool_fprop(const ng_pool_params* p, int dtype, int op,
  * depend on execution order.  Overlapping max pooling keeps one byte per output
  * element (the argmax slot) in `workspace`. */
 size_t ng_pool_workspace_bytes(const ng_pool_params* p, int dtype, int op);
+/* flags: 0, or NG_FLAG_RELU for max pooling over at most 255 elements when I is
+ * the output of a rectifier: gradI is additionally multiplied by (I > 0), the
+ * derivative step the layer below would apply next (`bprop_in *= fprop_out > 0`,
+ * nervanagpu/layers.py:89-91), at no extra memory traffic. */
 int ng_pool_bprop(const ng_pool_params* p, int dtype, int op,
-                  const void* I, const void* E, void* gradI,
+                  const void* I, const void* E, void* gradI, unsigned flags,
                   void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- small data-movement helpers ---------------------------------------------

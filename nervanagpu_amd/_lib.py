@@ -98,7 +98,7 @@ _SIGNATURES = {
                                c_float, c_void_p, c_size_t, c_void_p]),
     "ng_pool_fprop": (c_int, [POINTER(PoolParams), c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "ng_pool_workspace_bytes": (c_size_t, [POINTER(PoolParams), c_int, c_int]),
-    "ng_pool_bprop": (c_int, [POINTER(PoolParams), c_int, c_int, c_void_p, c_void_p, c_void_p,
+    "ng_pool_bprop": (c_int, [POINTER(PoolParams), c_int, c_int, c_void_p, c_void_p, c_void_p, c_uint,
                               c_void_p, c_size_t, c_void_p]),
     "ng_transpose": (c_int, [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "ng_dimshuffle": (c_int, [c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),

@@ -97,9 +97,14 @@ struct PoolGeom {
     // that hold at least one input element
     int use_cells, cells_h, cells_w, cell_remap;
     FastDiv div_ch, div_cw;
+    // max pooling backward with the rectifier derivative of the layer below
+    // folded in: a window whose maximum is not positive passes nothing on
+    int relu_mask;
 };
 
 enum { OP_MAX = 0, OP_AVG = 1 };
+// argmax value no element of a window of at most 255 elements carries
+enum { NO_SLOT = 255 };
 
 #define NG_FLT_MAX 3.402823466e+38f
 
@@ -228,6 +233,10 @@ void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char
                     for (int i = 0; i < VEC; i++)
                         slot_of[i] = (Lanes<T, VEC>::get(taps[tap], i) == Lanes<T, VEC>::get(top, i)) ? tap : slot_of[i];
                 }
+                if (g.relu_mask) {
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) slot_of[i] = ((float)Lanes<T, VEC>::get(top, i) > 0.0f) ? slot_of[i] : NO_SLOT;
+                }
                 store_slots<VEC>(arg + o, slot_of);
             }
             return;
@@ -272,6 +281,10 @@ void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char
     }
     const long o = ((long)k * per_map + inner) * VEC;
     if (WRITE_ARG) {
+        if (g.relu_mask) {
+#pragma unroll
+            for (int i = 0; i < VEC; i++) slot_of[i] = (best[i] > 0.0f) ? slot_of[i] : NO_SLOT;
+        }
         store_slots<VEC>(arg + o, slot_of);
     } else {
         if (OP == OP_AVG) {
@@ -529,6 +542,10 @@ void pool_bprop_max_tiled_kernel(const T* __restrict__ I, const T* __restrict__ 
                 if (v > best[i]) { best[i] = v; slot_of[i] = tap; }
             }
         }
+        if (g.relu_mask) {
+#pragma unroll
+            for (int i = 0; i < VEC; i++) slot_of[i] = (best[i] > 0.0f) ? slot_of[i] : NO_SLOT;
+        }
 #pragma unroll
         for (int tap = 0; tap < NTAP; tap++) {
             float out[VEC];
@@ -553,6 +570,10 @@ void pool_bprop_max_tiled_kernel(const T* __restrict__ I, const T* __restrict__ 
                     for (int i = 0; i < VEC; i++)
                         if (v[i] > best[i]) { best[i] = v[i]; slot_of[i] = slot; }
                 }
+    if (g.relu_mask) {
+#pragma unroll
+        for (int i = 0; i < VEC; i++) slot_of[i] = (best[i] > 0.0f) ? slot_of[i] : NO_SLOT;
+    }
     float ev[VEC];
     load_vec<T, VEC>(E + ((long)k * per_map + inner) * VEC, ev);
     slot = 0;
@@ -698,10 +719,11 @@ static void launch_gather(const PoolGeom& g, bool win2, dim3 grid, const T* E, c
 }
 
 template <typename T, int VEC>
-static int run_bprop(const ng_pool_params& p, int op, const void* I, const void* E, void* B,
+static int run_bprop(const ng_pool_params& p, int op, const void* I, const void* E, void* B, unsigned flags,
                      void* ws, size_t ws_bytes, hipStream_t st)
 {
     PoolGeom g = make_geom(p, VEC, sizeof(T));
+    g.relu_mask = (flags & NG_FLAG_RELU) ? 1 : 0;
     const long out_total = (long)g.K * g.M * g.P * g.Q * g.nvec;
     const dim3 out_grid = grid_for((long)g.M * g.P * g.Q * g.nvec, g.K, g.xcd_remap);
     const dim3 in_grid = grid_for((long)g.D * g.H * g.W * g.nvec, g.C);
@@ -763,19 +785,22 @@ int ng_pool_fprop(const ng_pool_params* p, int dtype, int op, const void* I, voi
 }
 
 int ng_pool_bprop(const ng_pool_params* p, int dtype, int op, const void* I, const void* E, void* gradI,
-                  void* workspace, size_t workspace_bytes, void* stream)
+                  unsigned flags, void* workspace, size_t workspace_bytes, void* stream)
 {
     int rc = check_params(*p, dtype, op);
     if (rc) return rc;
     if (!E || !gradI || (op == OP_MAX && !I)) return fail(-66, "pool: null tensor");
+    if (flags & ~(unsigned)NG_FLAG_RELU) return fail(-69, "pool bprop: unknown flag bits 0x%x", flags);
+    if ((flags & NG_FLAG_RELU) && (op != OP_MAX || p->J * p->T * p->R * p->S > 255))
+        return fail(-69, "pool bprop: the rectifier mask needs max pooling over windows of at most 255 elements");
     hipStream_t st = (hipStream_t)stream;
     const bool al = aligned16(E) && aligned16(gradI) && (op != OP_MAX || aligned16(I)) &&
                     (!workspace || aligned16(workspace));
     if (dtype == NG_F16)
-        return (al && p->N % 8 == 0) ? run_bprop<_Float16, 8>(*p, op, I, E, gradI, workspace, workspace_bytes, st)
-                                     : run_bprop<_Float16, 1>(*p, op, I, E, gradI, workspace, workspace_bytes, st);
-    return (al && p->N % 4 == 0) ? run_bprop<float, 4>(*p, op, I, E, gradI, workspace, workspace_bytes, st)
-                                 : run_bprop<float, 1>(*p, op, I, E, gradI, workspace, workspace_bytes, st);
+        return (al && p->N % 8 == 0) ? run_bprop<_Float16, 8>(*p, op, I, E, gradI, flags, workspace, workspace_bytes, st)
+                                     : run_bprop<_Float16, 1>(*p, op, I, E, gradI, flags, workspace, workspace_bytes, st);
+    return (al && p->N % 4 == 0) ? run_bprop<float, 4>(*p, op, I, E, gradI, flags, workspace, workspace_bytes, st)
+                                 : run_bprop<float, 1>(*p, op, I, E, gradI, flags, workspace, workspace_bytes, st);
 }
 
 }  // extern "C"

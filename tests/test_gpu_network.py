@@ -178,3 +178,40 @@ def test_inception_network_layerwise(ng, dtype):
         assert again is layer.bprop_out
         assert np.array_equal(again.get().view(np.uint8), first[0].view(np.uint8))
         propagation = again
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_relu_folded_into_pooling_gives_the_same_network(ng, dtype):
+    """fold_relu_into_pooling: the max pooling layers above rectified layers apply
+    the rectifier derivative themselves; every gradient of the network must equal
+    the reference flow's (separate elementwise pass)."""
+    from nervanagpu_amd import convnet_benchmarks as cb
+    from nervanagpu_amd.layers import PoolLayer
+
+    def run(fold):
+        layers = cb.build_network(ng, _small_net(), dtype, seed=5, fold_relu=fold)
+        for layer in layers:
+            layer.learning_rate = 0.0     # keep the weights of both runs identical
+        propagation = None
+        for layer in layers:
+            propagation = layer.fprop(propagation)
+        grads = []
+        for layer in layers[:0:-1]:
+            propagation = layer.bprop(propagation)
+            # a pooling layer's output differs by design (masked now, or by the
+            # layer below later, in place); what the rectified layers compute
+            # from it must not
+            if type(layer) is not PoolLayer:
+                grads.append(None if propagation is None else propagation.get().copy())
+                grads.append(layer.updat_out.get().copy())
+        return layers, grads
+
+    plain_layers, plain = run(False)
+    folded_layers, folded = run(True)
+    assert sum(bool(getattr(l, "relu_below", False)) for l in folded_layers) == 2
+    assert sum(l.relu_done_above for l in folded_layers) == 2 and not any(l.relu_done_above for l in plain_layers)
+    assert len(plain) == len(folded)
+    for a, b in zip(plain, folded):
+        assert (a is None) == (b is None)
+        if a is not None:
+            assert np.array_equal(a, b)

@@ -151,3 +151,46 @@ def test_pool_errors(ng):
         ng.fprop_pool(ok, ng.empty(layer.dimI), ng.empty((4, 1, 3, 3, 16)))
     with pytest.raises(AssertionError):
         ng.bprop_pool(ok, ng.empty(ok.dimI), ng.empty(ok.dimO), ng.empty(ok.dimI, dtype=np.float32))
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_max_pool_bprop_with_rectifier_mask(ng, dtype):
+    """bprop_pool(..., relu_mask=True) = bprop_pool followed by the reference's
+    relu derivative step `grad *= I > 0` (nervanagpu/layers.py:89-91), on every
+    backward path: exact tiling 2x2 and 3x3, generic exact tiling, overlapping
+    3x3/2 by cells, overlapping with padding, feature-map pooling, N = 4 lanes."""
+    rng = np.random.default_rng(23)
+    cases = [  # N, C, D, H, W, J, T, R, S, pads (j,d,h,w), strides (j,d,h,w)
+        (16, 6, 1, 8, 8, 1, 1, 2, 2, (0, 0, 0, 0), (1, 1, 2, 2)),
+        (16, 4, 1, 9, 9, 1, 1, 3, 3, (0, 0, 0, 0), (1, 1, 3, 3)),
+        (8, 4, 2, 8, 6, 1, 2, 2, 3, (0, 0, 0, 0), (1, 2, 2, 3)),
+        (16, 5, 1, 13, 13, 1, 1, 3, 3, (0, 0, 0, 0), (1, 1, 2, 2)),
+        (16, 3, 1, 12, 10, 1, 1, 3, 3, (0, 0, 1, 1), (1, 1, 2, 2)),
+        (8, 6, 1, 7, 7, 2, 1, 3, 3, (0, 0, 1, 1), (2, 1, 1, 1)),
+        (4, 3, 1, 9, 9, 1, 1, 3, 3, (0, 0, 0, 0), (1, 1, 2, 2)),
+    ]
+    for (N, C, D, H, W, J, T, R, S, pads, strides) in cases:
+        layer = ng.pool_layer(dtype, "max", N, C, D, H, W, J, T, R, S, *pads, *strides)
+        # about half of the inputs are zero (a rectifier's output), some windows entirely
+        x = np.maximum(rng.standard_normal(layer.dimI), 0).astype(dtype)
+        x[:, :, : H // 3, : W // 3, :] = 0
+        e = rng.uniform(-1, 1, layer.dimO).astype(dtype)
+        dI, dE = ng.array(x, dtype=dtype), ng.array(e, dtype=dtype)
+        plain, masked = ng.empty(layer.dimI, dtype=dtype), ng.empty(layer.dimI, dtype=dtype)
+        ng.bprop_pool(layer, dI, dE, plain)
+        ng.bprop_pool(layer, dI, dE, masked, relu_mask=True)
+        want = plain.get() * (x > 0)
+        assert np.array_equal(masked.get(), want), (N, C, D, H, W, J, T, R, S)
+        ref = orc.ref_pool_bprop(x.astype(np.float32), e.astype(np.float32), "max", layer.JTRS, layer.padding,
+                                 layer.strides) * (x > 0)
+        assert np.allclose(masked.get().astype(np.float32), ref.astype(dtype).astype(np.float32), rtol=2e-3, atol=1e-6)
+        # inputs that are not a rectifier's output: the mask is still (I > 0)
+        x2 = rng.standard_normal(layer.dimI).astype(dtype)
+        dI.set(x2)
+        ng.bprop_pool(layer, dI, dE, plain)
+        ng.bprop_pool(layer, dI, dE, masked, relu_mask=True)
+        assert np.array_equal(masked.get(), plain.get() * (x2 > 0))
+    avg = ng.pool_layer(np.float16, "avg", 16, 4, 1, 8, 8, 1, 1, 2, 2)
+    A, E, B = ng.empty(avg.dimI), ng.empty(avg.dimO), ng.empty(avg.dimI)
+    with pytest.raises(Exception):
+        ng.bprop_pool(avg, A, E, B, relu_mask=True)
