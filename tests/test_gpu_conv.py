@@ -25,6 +25,11 @@ SMALL = [
     (16, 144, 48, 1, 7, 7, 1, 1, 1, (0, 0, 0), (1, 1, 1)),        # 1x1 (inception style)
     (8, 96, 112, 1, 11, 10, 1, 3, 3, (0, 1, 1), (1, 2, 2)),       # strided, one launch per class
     (8, 48, 208, 1, 6, 6, 1, 2, 2, (0, 1, 1), (1, 1, 1)),
+    # one-dimensional filters with one-sided extents, depth stride with depth padding, a filter as large as the image
+    (8, 16, 24, 1, 9, 12, 1, 1, 7, (0, 0, 3), (1, 1, 1)),
+    (8, 16, 24, 1, 12, 9, 1, 7, 1, (0, 3, 0), (1, 1, 1)),
+    (8, 8, 8, 6, 7, 7, 3, 3, 3, (1, 1, 1), (2, 2, 2)),
+    (8, 8, 16, 1, 5, 5, 1, 5, 5, (0, 0, 0), (1, 1, 1)),
 ]
 
 
