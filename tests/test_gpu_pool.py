@@ -21,6 +21,10 @@ CASES = [
     (16, 3, 2, 12, 10, 1, 1, 3, 3, (0, 0, 0, 0), (1, 1, 2, 2)),      # 3x3/2 on even extents: last row / column uncovered
     (8, 4, 1, 7, 9, 1, 1, 3, 3, (0, 0, 1, 1), (1, 1, 2, 2)),         # 3x3/2 padded, odd non-square extents
     (4, 5, 1, 9, 11, 1, 1, 3, 3, (0, 0, 0, 1), (1, 1, 2, 2)),        # 3x3/2, four images: vector path only in fp32
+    (16, 6, 1, 10, 9, 1, 1, 3, 3, (0, 0, 1, 1), (1, 1, 1, 1)),       # 3x3/1 padded (inception pooling branch), vector path
+    (8, 10, 1, 5, 5, 3, 1, 1, 1, (1, 0, 0, 0), (2, 1, 1, 1)),        # overlapping, padded windows over feature maps
+    (8, 4, 7, 6, 6, 1, 3, 2, 2, (0, 1, 0, 0), (1, 2, 2, 2)),         # overlapping in depth only
+    (8, 3, 1, 9, 8, 1, 1, 2, 2, (0, 0, 0, 0), (1, 1, 1, 1)),         # 2x2/1: overlapping, no compiled cell shape
 ]
 
 
