@@ -158,9 +158,13 @@ int ng_conv_fprop(const void* plan, int in_dtype,
                   const void* I, const void* F, void* O, float alpha, unsigned flags,
                   void* workspace, size_t workspace_bytes, void* stream);
 /* gradI = round(alpha * conv_transpose(E, F)); deterministic gather form, every
- * element of gradI is written (no zero fill needed) */
+ * element of gradI is written (no zero fill needed).  relu_mask: NULL, or (unit
+ * strides only) the activations of the layer below, a tensor shaped like gradI:
+ * gradI is additionally multiplied by (relu_mask > 0), the derivative step that
+ * layer would apply next (`bprop_in *= fprop_out > 0`, nervanagpu/layers.py:89-91),
+ * for one read of the activations instead of an elementwise pass over both. */
 int ng_conv_bprop(const void* plan,
-                  const void* F, const void* E, void* gradI, float alpha,
+                  const void* F, const void* E, void* gradI, float alpha, const void* relu_mask,
                   void* workspace, size_t workspace_bytes, void* stream);
 /* gradF = round(alpha * sum_{pixels,n} I x E); out_dtype NG_F32 or NG_F16;
  * fp32 accumulation with a fixed-order reduction of the split partial sums */

@@ -93,7 +93,7 @@ _SIGNATURES = {
     "ng_conv_fprop": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                               c_float, c_uint, c_void_p, c_size_t, c_void_p]),
     "ng_conv_bprop": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p,
-                              c_float, c_void_p, c_size_t, c_void_p]),
+                              c_float, c_void_p, c_void_p, c_size_t, c_void_p]),
     "ng_conv_update": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                c_float, c_void_p, c_size_t, c_void_p]),
     "ng_pool_fprop": (c_int, [POINTER(PoolParams), c_int, c_int, c_void_p, c_void_p, c_void_p]),

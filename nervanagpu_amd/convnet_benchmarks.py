@@ -132,19 +132,25 @@ def network_config(name):
     return confs
 
 
-def fold_relu_into_pooling(layers):
-    """Where a max pooling layer directly follows a convolution or fully
-    connected layer, let the pooling backward kernel apply that layer's
-    rectifier derivative (it reads the same activations to find the maxima), so
-    the layer below skips its elementwise pass over the errors.  Same results;
-    not part of the reference's driver.  Returns the number of folded pairs."""
+def fold_relu_derivatives(layers):
+    """Let the backward kernel of the layer above apply a convolution or fully
+    connected layer's rectifier derivative, so that layer skips its elementwise
+    pass over the errors.  A max pooling layer above reads the same activations
+    to find its maxima (no extra traffic); a unit-stride convolution above
+    reads them once in its store.  Same results; not part of the reference's
+    driver.  Returns the number of folded pairs."""
     folded = 0
     for below, above in zip(layers[:-1], layers[1:]):
-        if (type(below) in (ConvLayer, FullLayer) and type(above) is PoolLayer and above.op == "max"
-                and reduce(mul, above.JTRS, 1) <= 255):
+        if type(below) not in (ConvLayer, FullLayer):
+            continue
+        if type(above) is PoolLayer and above.op == "max" and reduce(mul, above.JTRS, 1) <= 255:
             above.relu_below = True
-            below.relu_done_above = True
-            folded += 1
+        elif type(above) is ConvLayer and tuple(above.strides) == (1, 1, 1) and above.bprop_out is not None:
+            above.relu_mask_below = below.fprop_out
+        else:
+            continue
+        below.relu_done_above = True
+        folded += 1
     return folded
 
 
@@ -186,7 +192,7 @@ def build_network(ng, confs, dtype, zeros=False, seed=0, fold_relu=False):
             propagation = layer.fprop(propagation, scale_weights=.5)
         ng.bench = bench
     if fold_relu:
-        fold_relu_into_pooling(layers)
+        fold_relu_derivatives(layers)
     return layers
 
 
@@ -249,8 +255,9 @@ def main(argv=None):
     ap.add_argument("--quiet", action="store_true", help="only the per-network summary")
     ap.add_argument("--json", default=None, help="write the summaries to this file")
     ap.add_argument("--fold-relu", action="store_true",
-                    help="let max pooling backward apply the rectifier derivative of the layer below it "
-                         "(same results, one elementwise pass per such pair saved; not in the reference)")
+                    help="let max pooling and unit-stride convolution backward apply the rectifier derivative of "
+                         "the layer below them (same results, one elementwise pass per such pair saved; not in "
+                         "the reference)")
     args = ap.parse_args(argv)
     dtypes = {"f16": np.float16, "f32": np.float32}
     ng = NervanaGPU(stochastic_round=False, bench=False)

@@ -105,7 +105,7 @@ static int run_bprop_merged(const ConvPlan& pl, const void* F, const void* E, vo
 
 template <typename T, bool BLOCKED, int BM, int BN, int BK, int WM, int WN>
 static int bprop_class(const ConvPlan& pl, const BpropClass& c, const void* F, const T* Fs, const void* E, void* gradI,
-                       float alpha, hipStream_t stream)
+                       float alpha, const void* mask, hipStream_t stream)
 {
     const ng_conv_params& p = pl.p;
     const int ncols = c.nz * c.ny * c.nx * p.N;
@@ -119,7 +119,7 @@ static int bprop_class(const ConvPlan& pl, const BpropClass& c, const void* F, c
                                            BLOCKED ? c.taps : 0};
     const int k_tiles = cdiv(c.J, BK);
     const bool dense = (p.str_d == 1 && p.str_h == 1 && p.str_w == 1);
-    ScaleStoreEpilogue<T> depi{(T*)gradI, 0, ncols, p.C, ncols, alpha, 0.0f, 0u, 0u, 0u, 0u, 1u};
+    ScaleStoreEpilogue<T> depi{(T*)gradI, 0, ncols, p.C, ncols, alpha, 0.0f, 0u, 0u, 0u, 0u, 1u, (const T*)mask};
     LatticeStoreEpilogue<T> lepi{(T*)gradI, p.C, (long)p.D * p.H * p.W * p.N, lat, c.rz, c.ry, c.rx,
                                  p.str_d, p.str_h, p.str_w, p.H, p.W, alpha};
     if constexpr (BLOCKED) {
@@ -137,20 +137,23 @@ static int bprop_class(const ConvPlan& pl, const BpropClass& c, const void* F, c
 
 template <bool BLOCKED>
 static int bprop_class_h(const ConvPlan& pl, const BpropClass& c, const void* F, const _Float16* Fs, const void* E,
-                         void* gradI, float alpha, hipStream_t st)
+                         void* gradI, float alpha, const void* mask, hipStream_t st)
 {
     switch (pick_row_tile(pl.p.C, c.nz * c.ny * c.nx * pl.p.N, 256)) {
-    case 256: return bprop_class<_Float16, BLOCKED, 256, 256, 64, 2, 4>(pl, c, F, Fs, E, gradI, alpha, st);
-    case 128: return bprop_class<_Float16, BLOCKED, 128, 256, 64, 2, 4>(pl, c, F, Fs, E, gradI, alpha, st);
-    default:  return bprop_class<_Float16, BLOCKED, 64, 256, 64, 1, 4>(pl, c, F, Fs, E, gradI, alpha, st);
+    case 256: return bprop_class<_Float16, BLOCKED, 256, 256, 64, 2, 4>(pl, c, F, Fs, E, gradI, alpha, mask, st);
+    case 128: return bprop_class<_Float16, BLOCKED, 128, 256, 64, 2, 4>(pl, c, F, Fs, E, gradI, alpha, mask, st);
+    default:  return bprop_class<_Float16, BLOCKED, 64, 256, 64, 1, 4>(pl, c, F, Fs, E, gradI, alpha, mask, st);
     }
 }
 
 template <typename T>
-static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gradI, float alpha,
+static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gradI, float alpha, const void* mask,
                      void* ws, size_t ws_bytes, hipStream_t stream)
 {
     const ng_conv_params& p = pl.p;
+    // the mask shares the plain store epilogue's indexing: unit strides only
+    if (mask && (pl.merged || p.str_d != 1 || p.str_h != 1 || p.str_w != 1))
+        return fail(-51, "ng_conv_bprop: the rectifier mask needs unit strides");
     if (pl.ws_bprop && (ws_bytes < pl.ws_bprop || !ws))
         return fail(-40, "ng_conv_bprop: workspace too small (%zu < %zu)", ws_bytes, pl.ws_bprop);
     if (pl.merged)
@@ -169,11 +172,11 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
         if (c.nz * c.ny * c.nx == 0) continue;
         int rc;
         if (sizeof(T) == 2)
-            rc = blocked ? bprop_class_h<true>(pl, c, F, (const _Float16*)Fs, E, gradI, alpha, stream)
-                         : bprop_class_h<false>(pl, c, F, (const _Float16*)Fs, E, gradI, alpha, stream);
+            rc = blocked ? bprop_class_h<true>(pl, c, F, (const _Float16*)Fs, E, gradI, alpha, mask, stream)
+                         : bprop_class_h<false>(pl, c, F, (const _Float16*)Fs, E, gradI, alpha, mask, stream);
         else
-            rc = blocked ? bprop_class<float, true, 128, 128, 16, 2, 2>(pl, c, F, (const float*)Fs, E, gradI, alpha, stream)
-                         : bprop_class<float, false, 128, 128, 16, 2, 2>(pl, c, F, (const float*)Fs, E, gradI, alpha, stream);
+            rc = blocked ? bprop_class<float, true, 128, 128, 16, 2, 2>(pl, c, F, (const float*)Fs, E, gradI, alpha, mask, stream)
+                         : bprop_class<float, false, 128, 128, 16, 2, 2>(pl, c, F, (const float*)Fs, E, gradI, alpha, mask, stream);
         if (rc) return rc;
     }
     return 0;
@@ -184,15 +187,16 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
 using namespace ng;
 
 extern "C" int ng_conv_bprop(const void* plan, const void* F, const void* E, void* gradI, float alpha,
-                             void* workspace, size_t workspace_bytes, void* stream)
+                             const void* relu_mask, void* workspace, size_t workspace_bytes, void* stream)
 {
     const ConvPlan* pl = (const ConvPlan*)plan;
     if (!pl) return fail(-48, "conv: null plan");
     int rc;
     if ((rc = check_ptr16(F, "F")) || (rc = check_ptr16(E, "E")) || (rc = check_ptr16(gradI, "grad_I")) ||
+        (relu_mask && (rc = check_ptr16(relu_mask, "relu_mask"))) ||
         (pl->ws_bprop && (rc = check_ptr16(workspace, "workspace"))))
         return rc;
     hipStream_t st = (hipStream_t)stream;
-    if (pl->dtype == NG_F16) return run_bprop<_Float16>(*pl, F, E, gradI, alpha, workspace, workspace_bytes, st);
-    return run_bprop<float>(*pl, F, E, gradI, alpha, workspace, workspace_bytes, st);
+    if (pl->dtype == NG_F16) return run_bprop<_Float16>(*pl, F, E, gradI, alpha, relu_mask, workspace, workspace_bytes, st);
+    return run_bprop<float>(*pl, F, E, gradI, alpha, relu_mask, workspace, workspace_bytes, st);
 }

@@ -941,6 +941,26 @@ struct ScaleStoreEpilogue {
     unsigned relu;
     unsigned sr_bits, seed, stream;
     unsigned vec;   // rows of C are 16-byte aligned and n is a multiple of 8
+    // optional tensor laid out like C (16-byte aligned): outputs whose mask
+    // element is not positive are stored as zero (the rectifier derivative of
+    // the layer whose activations the mask holds)
+    const T* mask = nullptr;
+
+    __device__ __forceinline__ bool masked_out(long offset) const
+    {
+        return !(StoreBits<T>::widen(reinterpret_cast<const bits_t*>(mask)[offset]) > 0.0f);
+    }
+    // zero those of 8 consecutive outputs at element offset `offset` whose mask is not positive
+    __device__ __forceinline__ void mask8(bits_t (&out)[8], long offset) const
+    {
+        constexpr int NV = (int)sizeof(bits_t) * 8 / 16;
+        bits_t mk[8];
+#pragma unroll
+        for (int q = 0; q < NV; q++)
+            reinterpret_cast<uint4_t*>(mk)[q] = reinterpret_cast<const uint4_t*>(reinterpret_cast<const bits_t*>(mask) + offset)[q];
+#pragma unroll
+        for (int e = 0; e < 8; e++) out[e] = (StoreBits<T>::widen(mk[e]) > 0.0f) ? out[e] : (bits_t)0;
+    }
 
     __device__ __forceinline__ float scale(float acc) const
     {
@@ -954,15 +974,18 @@ struct ScaleStoreEpilogue {
     __device__ __forceinline__ void apply(int i, int j, int z, float acc) const
     {
         float v = scale(acc);
-        bits_t* p = reinterpret_cast<bits_t*>(C + (long)z * ldcz + (long)i * ldc + j);
+        const long offset = (long)z * ldcz + (long)i * ldc + j;
+        bits_t* p = reinterpret_cast<bits_t*>(C + offset);
         if (beta != 0.0f) v += beta * StoreBits<T>::widen(*p);
-        *p = StoreBits<T>::round(v, sr_bits, seed, stream, rng_index(i, j, z));
+        const bits_t r = StoreBits<T>::round(v, sr_bits, seed, stream, rng_index(i, j, z));
+        *p = (mask && masked_out(offset)) ? (bits_t)0 : r;
     }
     __device__ __forceinline__ void store8(int i, int j0, int z, int /*split*/, const float (&acc)[8]) const
     {
         if (i >= m || j0 >= n) return;
         constexpr int NV = (int)sizeof(bits_t) * 8 / 16;   // 16-byte pieces per 8 elements
-        bits_t* p = reinterpret_cast<bits_t*>(C + (long)z * ldcz + (long)i * ldc + j0);
+        const long offset = (long)z * ldcz + (long)i * ldc + j0;
+        bits_t* p = reinterpret_cast<bits_t*>(C + offset);
         if (vec && beta == 0.0f && sr_bits == 0) {
             // common case, kept free of the rounding-stream arithmetic:
             // scale, optional relu, nearest rounding, 16-byte stores
@@ -970,6 +993,7 @@ struct ScaleStoreEpilogue {
             bits_t out[8];
 #pragma unroll
             for (int e = 0; e < 8; e++) out[e] = StoreBits<T>::round(fmaxf(acc[e] * alpha, lo), 0, 0, 0, 0);
+            if (mask) mask8(out, offset);
 #pragma unroll
             for (int q = 0; q < NV; q++)
                 reinterpret_cast<uint4_t*>(p)[q] = reinterpret_cast<const uint4_t*>(out)[q];
@@ -987,6 +1011,12 @@ struct ScaleStoreEpilogue {
                     v1 += beta * StoreBits<T>::widen(cur[2 * q + 1]);
                 }
                 packed[q] = ng_sr10_f16x2(v0, v1, ng_rand32(seed, stream, pair0 + q));
+            }
+            if (mask) {
+                bits_t out[8];
+                *reinterpret_cast<uint4_t*>(out) = *reinterpret_cast<const uint4_t*>(packed);
+                mask8(out, offset);
+                *reinterpret_cast<uint4_t*>(packed) = *reinterpret_cast<const uint4_t*>(out);
             }
             *reinterpret_cast<uint4_t*>(p) = *reinterpret_cast<const uint4_t*>(packed);
         } else if (vec) {
@@ -1006,6 +1036,7 @@ struct ScaleStoreEpilogue {
                 if (beta != 0.0f) v += beta * StoreBits<T>::widen(out[e]);
                 out[e] = sr_bits ? StoreBits<T>::round_word(v, sr_bits, words[e]) : StoreBits<T>::round(v, 0, 0, 0, 0);
             }
+            if (mask) mask8(out, offset);
 #pragma unroll
             for (int q = 0; q < NV; q++)
                 reinterpret_cast<uint4_t*>(p)[q] = reinterpret_cast<const uint4_t*>(out)[q];

@@ -245,3 +245,32 @@ def test_deconv_layer_and_errors(ng):
         ng.fprop_conv(small, ng.empty((3, 1, 8, 8, 8)), ng.empty(small.dimF), ng.empty(small.dimO))
     with pytest.raises(AssertionError):
         ng.fprop_conv(small, ng.empty(small.dimI), ng.empty(small.dimF, dtype=np.float32), ng.empty(small.dimO))
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_bprop_with_rectifier_mask(ng, dtype):
+    """bprop_conv(..., relu_mask=act) = bprop_conv followed by the reference's
+    relu derivative step `grad *= act > 0` (nervanagpu/layers.py:89-91), on the
+    blocked and the row-by-row form, full and ragged tiles; strided layers refuse."""
+    rng = np.random.default_rng(29)
+    for case in (SMALL[0], SMALL[2], SMALL[5], SMALL[8], SMALL[11], (16, 64, 64, 1, 20, 20, 1, 3, 3, (0, 1, 1), (1, 1, 1))):
+        layer = _layer(ng, dtype, case)
+        I, F, E = _data(layer, dtype, 31)
+        act = np.maximum(rng.standard_normal(layer.dimI), 0).astype(dtype)     # about half zeros
+        dF, dE, dA = ng.array(F, dtype=dtype), ng.array(E, dtype=dtype), ng.array(act, dtype=dtype)
+        plain, masked = ng.empty(layer.dimI, dtype=dtype), ng.empty(layer.dimI, dtype=dtype)
+        ng.bprop_conv(layer, dF, dE, plain)
+        masked.fill(7)
+        ng.bprop_conv(layer, dF, dE, masked, relu_mask=dA)
+        assert np.array_equal(masked.get(), plain.get() * (act > 0)), case
+        # a mask with negative entries and negative zeros: only > 0 passes
+        act2 = rng.standard_normal(layer.dimI).astype(dtype)
+        act2[..., ::3] = -0.0
+        dA.set(act2)
+        ng.bprop_conv(layer, dF, dE, masked, relu_mask=dA)
+        assert np.array_equal(masked.get(), plain.get() * (act2 > 0)), case
+    strided = _layer(ng, dtype, SMALL[7])
+    I, F, E = _data(strided, dtype, 31)
+    out = ng.empty(strided.dimI, dtype=dtype)
+    with pytest.raises(Exception):
+        ng.bprop_conv(strided, ng.array(F, dtype=dtype), ng.array(E, dtype=dtype), out, relu_mask=ng.empty(strided.dimI, dtype=dtype))

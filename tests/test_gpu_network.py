@@ -180,36 +180,50 @@ def test_inception_network_layerwise(ng, dtype):
         propagation = again
 
 
+def _conv_pairs_net():
+    from nervanagpu_amd.layers import DataLayer, ConvLayer, PoolLayer, FullLayer
+    return [
+        {"layer": DataLayer, "N": 16, "C": 3, "H": 16, "W": 16},
+        {"layer": ConvLayer, "K": 16, "R": 3, "S": 3, "pad_h": 1, "pad_w": 1},
+        {"layer": ConvLayer, "K": 24, "R": 3, "S": 3, "pad_h": 1, "pad_w": 1},
+        {"layer": PoolLayer, "op": "max", "R": 2, "S": 2},
+        {"layer": ConvLayer, "K": 32, "R": 3, "S": 3, "pad_h": 1, "pad_w": 1},
+        {"layer": ConvLayer, "K": 32, "R": 1, "S": 1},
+        {"layer": ConvLayer, "K": 16, "R": 3, "S": 3, "str_h": 2, "str_w": 2},   # strided: not folded
+        {"layer": PoolLayer, "op": "avg", "R": 3, "S": 3},                       # average: not folded
+        {"layer": FullLayer, "nOut": 16},
+    ]
+
+
+@pytest.mark.parametrize("net,pairs", [(_small_net, 2), (_conv_pairs_net, 3)])
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
-def test_relu_folded_into_pooling_gives_the_same_network(ng, dtype):
-    """fold_relu_into_pooling: the max pooling layers above rectified layers apply
-    the rectifier derivative themselves; every gradient of the network must equal
-    the reference flow's (separate elementwise pass)."""
+def test_folded_rectifier_derivatives_give_the_same_network(ng, dtype, net, pairs):
+    """fold_relu_derivatives: max pooling and unit-stride convolution layers above
+    rectified layers apply the rectifier derivative themselves; every gradient the
+    rectified layers compute must equal the reference flow's (separate
+    elementwise pass)."""
     from nervanagpu_amd import convnet_benchmarks as cb
     from nervanagpu_amd.layers import PoolLayer
 
     def run(fold):
-        layers = cb.build_network(ng, _small_net(), dtype, seed=5, fold_relu=fold)
-        for layer in layers:
-            layer.learning_rate = 0.0     # keep the weights of both runs identical
+        layers = cb.build_network(ng, net(), dtype, seed=5, fold_relu=fold)
         propagation = None
         for layer in layers:
             propagation = layer.fprop(propagation)
         grads = []
         for layer in layers[:0:-1]:
             propagation = layer.bprop(propagation)
-            # a pooling layer's output differs by design (masked now, or by the
-            # layer below later, in place); what the rectified layers compute
-            # from it must not
-            if type(layer) is not PoolLayer:
-                grads.append(None if propagation is None else propagation.get().copy())
+            # what a layer hands down differs by design (masked now, or by the
+            # layer below later, in place); what the layer below computes from
+            # it must not: weight gradients, and data gradients after masking
+            if layer.weights is not None:
                 grads.append(layer.updat_out.get().copy())
+        grads.append(None if propagation is None else propagation.get().copy())
         return layers, grads
 
     plain_layers, plain = run(False)
     folded_layers, folded = run(True)
-    assert sum(bool(getattr(l, "relu_below", False)) for l in folded_layers) == 2
-    assert sum(l.relu_done_above for l in folded_layers) == 2 and not any(l.relu_done_above for l in plain_layers)
+    assert sum(l.relu_done_above for l in folded_layers) == pairs and not any(l.relu_done_above for l in plain_layers)
     assert len(plain) == len(folded)
     for a, b in zip(plain, folded):
         assert (a is None) == (b is None)
