@@ -156,14 +156,32 @@ def cpu_baseline(cases):
 # --all: every configured case with its own roofline
 # ---------------------------------------------------------------------------
 
+def cpu_seconds(fn, repeats=2):
+    """best wall time of the oracle call fn() after one untimed first touch"""
+    fn()
+    best = None
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        fn()
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    return best
+
+
+CPU_SAMPLE_PIXELS = 48      # output pixels per convolution layer timed on the CPU
+CPU_SAMPLE_WINDOWS = 2048   # pooling windows timed on the CPU
+
 ALEXNET = [(3, 224, 224, 64, 11, 11, 4, 2), (64, 27, 27, 192, 5, 5, 1, 2), (192, 13, 13, 384, 3, 3, 1, 1),
            (384, 13, 13, 256, 3, 3, 1, 1), (256, 13, 13, 256, 3, 3, 1, 1)]
 VGG = [(3, 224, 64), (64, 224, 64), (64, 112, 128), (128, 112, 128), (128, 56, 256), (256, 56, 256),
        (256, 28, 512), (512, 28, 512), (512, 14, 512)]
 
 
-def row(name, ms, flops=None, nbytes=None, peak_tflops=PEAK_FP16_TFLOPS):
+def row(name, ms, flops=None, nbytes=None, peak_tflops=PEAK_FP16_TFLOPS, cpu=None):
+    """cpu: (rate, unit, sample) of the numpy oracle on the host for the same case"""
     r = {"case": name, "ms": ms}
+    if cpu:
+        r["cpu_rate"], r["cpu_unit"], r["cpu_sample"] = cpu
     if flops:
         tf = flops / ms / 1e9
         r["tflops"] = tf
@@ -178,7 +196,21 @@ def row(name, ms, flops=None, nbytes=None, peak_tflops=PEAK_FP16_TFLOPS):
     return r
 
 
-def conv_rows(ng, tag, N, layers, rows, iters):
+def conv_cpu(layer, rng):
+    """the oracle's per-pixel gather + np.dot on a random sample of output pixels,
+    scaled to the layer: (TFLOP/s, unit, sample)"""
+    import oracle as orc
+    M, P, Q = layer.MPQ
+    I = np.full(layer.dimI, 0.5, dtype=np.float16)
+    F = rng.standard_normal(layer.dimF).astype(np.float16)
+    pixels = [(int(rng.integers(M)), int(rng.integers(P)), int(rng.integers(Q))) for _ in range(CPU_SAMPLE_PIXELS)]
+    sec = cpu_seconds(lambda: orc.ref_conv_fprop_pixels(I, F, pixels, layer.padding, layer.strides, relu=True,
+                                                        acc_dtype=np.float32), repeats=1)
+    flops = layer.flops * len(pixels) / float(M * P * Q)
+    return (flops / sec / 1e12, "TFLOP/s", "%d of %d output pixels" % (len(pixels), M * P * Q))
+
+
+def conv_rows(ng, tag, N, layers, rows, iters, cpu=False):
     rng = np.random.default_rng(2)
     for cfg in layers:
         if tag == "conv3d":
@@ -202,7 +234,7 @@ def conv_rows(ng, tag, N, layers, rows, iters):
         sI, sF, sO = layer.sizeI * 2, layer.sizeF * 2, layer.sizeO * 2
         nm = "%s C%d K%d %s %s" % (tag, layer.C, layer.K, layer.DHW, layer.TRS)
         ms = time_gpu(ng, lambda: ng.fprop_conv(layer, I, F, O, relu=True), iters)
-        rows.append(row(nm + " fprop", ms, layer.flops, sI + sF + sO))
+        rows.append(row(nm + " fprop", ms, layer.flops, sI + sF + sO, cpu=conv_cpu(layer, rng) if cpu else None))
         if tag != "conv3d":
             ms = time_gpu(ng, lambda: ng.bprop_conv(layer, F, E, B), iters)
             rows.append(row(nm + " bprop", ms, layer.flops, sI + sF + sO))
@@ -211,7 +243,22 @@ def conv_rows(ng, tag, N, layers, rows, iters):
         del I, F, E, O, B, U
 
 
-def pool_rows(ng, tag, N, C, HW, win, strd, op, rows, iters):
+def pool_cpu(layer, nbytes):
+    """the oracle's gather + np.max / np.mean on a random sample of windows,
+    scaled to the layer's algorithmic bytes: (GB/s, unit, sample)"""
+    import oracle as orc
+    rng = np.random.default_rng(3)
+    K, M, P, Q = layer.K, layer.MPQ[0], layer.MPQ[1], layer.MPQ[2]
+    I = np.full(layer.dimI, 0.5, dtype=np.float16)
+    windows = [(int(rng.integers(K)), int(rng.integers(M)), int(rng.integers(P)), int(rng.integers(Q)))
+               for _ in range(CPU_SAMPLE_WINDOWS)]
+    sec = cpu_seconds(lambda: orc.ref_pool_fprop_pixels(I, layer.op, layer.JTRS, windows, layer.padding, layer.strides),
+                      repeats=1)
+    total = K * M * P * Q
+    return (nbytes * len(windows) / float(total) / sec / 1e9, "GB/s", "%d of %d windows" % (len(windows), total))
+
+
+def pool_rows(ng, tag, N, C, HW, win, strd, op, rows, iters, cpu=False):
     layer = ng.pool_layer(np.float16, op, N, C, 1, HW, HW, 1, 1, win, win, 0, 0, 0, 0, 1, 1, strd, strd)
     I = ng.empty(layer.dimI)
     E = ng.empty(layer.dimO)
@@ -222,30 +269,39 @@ def pool_rows(ng, tag, N, C, HW, win, strd, op, rows, iters):
     sI, sO = layer.sizeI * 2, layer.sizeO * 2
     nm = "%s %s %dx%d/%d C%d %dx%d N%d" % (tag, op, win, win, strd, C, HW, HW, N)
     ms = time_gpu(ng, lambda: ng.fprop_pool(layer, I, O), iters)
-    rows.append(row(nm + " fprop", ms, None, sI + sO))
+    rows.append(row(nm + " fprop", ms, None, sI + sO, cpu=pool_cpu(layer, sI + sO) if cpu else None))
     ms = time_gpu(ng, lambda: ng.bprop_pool(layer, I, E, B), iters)
     rows.append(row(nm + " bprop", ms, None, (2 * sI + sO) if op == "max" else (sI + sO)))
 
 
-def all_cases(ng, cases, iters=10):
+def all_cases(ng, cases, iters=10, cpu=False):
+    """cpu: also time the numpy oracle on the host for one case of every kind
+    (np.dot for the GEMMs, sampled pixels / windows for convolution and pooling
+    forward, the whole array for the elementwise cases)"""
     from nervanagpu_amd import NervanaGPU
+    import oracle as orc
     rows = []
+
+    def gemm_cpu(c):
+        if not cpu:
+            return None
+        return (c.flops / cpu_seconds(c.cpu, repeats=1) / 1e12, "TFLOP/s", "np.dot, fp32 BLAS, %d threads" % blas_threads())
     # config 1
     for op in ("nn", "tn"):
         c = GemmCase(ng, op, 1024, 1024, 1024, dtype=np.float32, seed=0)
-        rows.append(row("cfg1 " + c.name(), time_gpu(ng, c.run, iters), c.flops, c.bytes, PEAK_FP32_TFLOPS))
+        rows.append(row("cfg1 " + c.name(), time_gpu(ng, c.run, iters), c.flops, c.bytes, PEAK_FP32_TFLOPS, cpu=gemm_cpu(c)))
     # config 2
     for c in cases:
         if c.relu or c.sr:
             continue
-        rows.append(row("cfg2 " + c.name(), time_gpu(ng, c.run, iters), c.flops, c.bytes))
+        rows.append(row("cfg2 " + c.name(), time_gpu(ng, c.run, iters), c.flops, c.bytes, cpu=gemm_cpu(c)))
     for c in cases:
         if c.sr and c.relu and c.op == "nn":
             rows.append(row("cfg2 " + c.name(), time_gpu(ng, c.run, iters), c.flops, c.bytes))
-    conv_rows(ng, "cfg3 alexnet", 128, ALEXNET, rows, iters)
-    conv_rows(ng, "cfg4 vgg", 64, VGG, rows, iters)
+    conv_rows(ng, "cfg3 alexnet", 128, ALEXNET, rows, iters, cpu)
+    conv_rows(ng, "cfg4 vgg", 64, VGG, rows, iters, cpu)
     for (C, HW) in ((64, 224), (128, 112), (256, 56), (512, 28), (512, 14)):
-        pool_rows(ng, "cfg4", 64, C, HW, 2, 2, "max", rows, iters)
+        pool_rows(ng, "cfg4", 64, C, HW, 2, 2, "max", rows, iters, cpu)
     # config 5
     ngs = NervanaGPU(stochastic_round=True, seed=4)
     A = ngs.empty((4096, 8192))
@@ -253,27 +309,36 @@ def all_cases(ng, cases, iters=10):
 
     def bn():
         A[:] = (A - ngs.mean(A, axis=1)) / ngs.sqrt(ngs.var(A, axis=1) + 1e-3)
-    rows.append(row("cfg5 batchnorm (4096,8192) fp16 SR", time_gpu(ngs, bn, iters), None, 2 * A.nbytes))
+    hA = np.random.default_rng(4).uniform(0, 1, (4096, 8192)).astype(np.float16) if cpu else None
+    bn_cpu = ew_cpu = None
+    if cpu:
+        sec = cpu_seconds(lambda: orc.ref_batchnorm_rows(hA, 1e-3).astype(np.float16), repeats=1)
+        bn_cpu = (2 * hA.nbytes / sec / 1e9, "GB/s", "numpy, whole array")
+        h32 = hA.astype(np.float32)
+        sec = cpu_seconds(lambda: (h32 * h32 + h32).astype(np.float16), repeats=1)
+        ew_cpu = (2 * hA.nbytes / sec / 1e9, "GB/s", "numpy, whole array")
+    rows.append(row("cfg5 batchnorm (4096,8192) fp16 SR", time_gpu(ngs, bn, iters), None, 2 * A.nbytes, cpu=bn_cpu))
     Bt = ngs.empty((4096, 8192))
     rows.append(row("cfg5 elementwise a*b+c (4096,8192) fp16",
-                    time_gpu(ngs, lambda: Bt._assign(A * A + A), iters), None, 2 * A.nbytes))
+                    time_gpu(ngs, lambda: Bt._assign(A * A + A), iters), None, 2 * A.nbytes, cpu=ew_cpu))
     for op in ("max", "avg"):
-        pool_rows(ng, "cfg5", 128, 256, 56, 3, 2, op, rows, iters)
-    conv_rows(ng, "conv3d", 32, [(64, 16, 28, 28, 128, 3, 3, 3)], rows, iters)
+        pool_rows(ng, "cfg5", 128, 256, 56, 3, 2, op, rows, iters, cpu)
+    conv_rows(ng, "conv3d", 32, [(64, 16, 28, 28, 128, 3, 3, 3)], rows, iters, cpu)
     return rows
 
 
 def format_rows(rows):
-    lines = ["| case | GPU ms | TFLOP/s | % MFMA peak | % of min(MFMA, AI*BW) | GB/s | % HBM peak |",
-             "|---|---|---|---|---|---|---|"]
+    lines = ["| case | GPU ms | TFLOP/s | % MFMA peak | % of min(MFMA, AI*BW) | GB/s | % HBM peak | CPU oracle |",
+             "|---|---|---|---|---|---|---|---|"]
     for r in rows:
-        lines.append("| %s | %.4f | %s | %s | %s | %s | %s |" % (
+        lines.append("| %s | %.4f | %s | %s | %s | %s | %s | %s |" % (
             r["case"], r["ms"],
             "%.1f" % r["tflops"] if "tflops" in r else "",
             "%.1f" % r["pct_mfma_peak"] if "pct_mfma_peak" in r else "",
             "%.1f" % r["pct_of_min_roof"] if "pct_of_min_roof" in r else "",
             "%.0f" % r["gbs"] if "gbs" in r else "",
-            "%.1f" % r["pct_hbm_peak"] if "pct_hbm_peak" in r else ""))
+            "%.1f" % r["pct_hbm_peak"] if "pct_hbm_peak" in r else "",
+            "%.3g %s (%s)" % (r["cpu_rate"], r["cpu_unit"], r["cpu_sample"]) if "cpu_rate" in r else ""))
     return "\n".join(lines)
 
 
@@ -365,7 +430,7 @@ def main():
         result["cpu_baseline"] = cpu_baseline(cases)
 
     if args.all:
-        rows = all_cases(ng, cases)
+        rows = all_cases(ng, cases, cpu=not args.no_cpu)
         table = format_rows(rows)
         if args.out:
             with open(args.out, "w") as f:
