@@ -137,7 +137,7 @@ VGG = [  # C,HW,K at N=64, 3x3 s1 p1 (benchmark configuration 4)
     (256, 28, 512), (512, 28, 512), (512, 14, 512)]
 
 
-def _sampled_layer_check(ng, layer, seed, gen, npix=24, nrows=6, in_dtype=np.float16):
+def _sampled_layer_check(ng, layer, seed, gen, npix=256, nrows=6, in_dtype=np.float16):
     rng = np.random.default_rng(seed)
     I, F, E = gen(rng, layer)
     dI = ng.array(I, dtype=in_dtype)
@@ -149,9 +149,19 @@ def _sampled_layer_check(ng, layer, seed, gen, npix=24, nrows=6, in_dtype=np.flo
     scale_i, scale_f, scale_e = np.abs(If).max(), np.abs(F.astype(np.float32)).max(), np.abs(E.astype(np.float32)).max()
 
     def sample(dims):
+        """npix random positions, the corners of the volume, and positions on
+        every face (first / last index of one coordinate, the others random):
+        the places where padding and ragged tiles show"""
         pts = [tuple(int(rng.integers(0, d)) for d in dims) for _ in range(npix)]
-        pts += [tuple(0 for _ in dims), tuple(d - 1 for d in dims), (0, 0, dims[2] - 1), (0, dims[1] - 1, 0)]
-        return pts
+        pts += [tuple(0 for _ in dims), tuple(d - 1 for d in dims), (0, 0, dims[2] - 1), (0, dims[1] - 1, 0),
+                (dims[0] - 1, 0, 0), (dims[0] - 1, dims[1] - 1, 0), (dims[0] - 1, 0, dims[2] - 1), (0, dims[1] - 1, dims[2] - 1)]
+        for axis in range(3):
+            for edge in (0, dims[axis] - 1):
+                for _ in range(3):
+                    pt = [int(rng.integers(0, d)) for d in dims]
+                    pt[axis] = edge
+                    pts.append(tuple(pt))
+        return sorted(set(pts))
 
     dO = ng.empty(layer.dimO)
     ng.fprop_conv(layer, dI, dF, dO, relu=True)
@@ -193,7 +203,7 @@ def _alexnet_data(rng, layer):
 def test_config3_alexnet_layers(ng, cfg):
     C, H, W, K, R, S, strd, pad = cfg
     layer = ng.conv_layer(np.float16, 128, C, K, 1, H, W, 1, R, S, 0, pad, pad, 1, strd, strd)
-    _sampled_layer_check(ng, layer, 2, _alexnet_data, npix=12 if C * R * S > 2000 else 24)
+    _sampled_layer_check(ng, layer, 2, _alexnet_data, npix=256)
 
 
 def test_config3_first_layer_uint8(ng):
@@ -218,7 +228,7 @@ def test_config4_vgg_layers(ng, cfg):
         F = (rng.standard_normal(layer.dimF) * np.sqrt(2.0 / (C * 9))).astype(np.float16)
         E = rng.standard_normal(layer.dimO, dtype=np.float32).astype(np.float16)
         return I, F, E
-    _sampled_layer_check(ng, layer, 3, gen, npix=10, nrows=3)
+    _sampled_layer_check(ng, layer, 3, gen, npix=256, nrows=4)
 
 
 def test_config5_conv3d(ng):
@@ -230,7 +240,7 @@ def test_config5_conv3d(ng):
         F = (rng.standard_normal(layer.dimF) * 0.05).astype(np.float16)
         E = rng.uniform(-1, 1, layer.dimO).astype(np.float16)
         return I, F, E
-    _sampled_layer_check(ng, layer, 4, gen, npix=10, nrows=3)
+    _sampled_layer_check(ng, layer, 4, gen, npix=256, nrows=4)
 
 
 def test_deconv_layer_and_errors(ng):
