@@ -102,10 +102,11 @@ def test_max_pool_negative_inputs_padding_and_signed_zero_ties(ng, dtype):
 
 
 def test_config4_vgg_pool_shapes(ng):
-    """2x2/2 max pooling at the five block ends of config 4 (reduced in C to bound
-    host time, full in H, W, N); idempotent structure: pooled gradient sums match"""
+    """2x2/2 max pooling at the five block ends of config 4, full shapes, every
+    element: the forward result against a reshape + max, and the structure of
+    the backward result (each window passes its error to exactly one element)"""
     rng = np.random.default_rng(3)
-    for C, HW in ((8, 224), (8, 112), (16, 56), (32, 28), (64, 14)):
+    for C, HW in ((64, 224), (128, 112), (256, 56), (512, 28), (512, 14)):
         layer = ng.pool_layer(np.float16, "max", 64, C, 1, HW, HW, 1, 1, 2, 2)
         I = rng.standard_normal(layer.dimI, dtype=np.float32).astype(np.float16)
         E = rng.standard_normal(layer.dimO, dtype=np.float32).astype(np.float16)
@@ -115,10 +116,15 @@ def test_config4_vgg_pool_shapes(ng):
         ng.bprop_pool(layer, dI, dE, dB)
         ref = I.astype(np.float32).reshape(C, 1, HW // 2, 2, HW // 2, 2, 64).max(axis=(3, 5))
         assert np.array_equal(dO.get(), ref.astype(np.float16))
+        del ref
         B = dB.get().astype(np.float32)
-        # each window passes its error to exactly one element
+        # each window passes its error to exactly one element: the first maximum
         assert np.array_equal(B.reshape(C, 1, HW // 2, 2, HW // 2, 2, 64).sum(axis=(3, 5)), E.astype(np.float32))
         assert np.count_nonzero(B) <= E.size
+        If = I.astype(np.float32)
+        at_max = If == np.repeat(np.repeat(dO.get().astype(np.float32), 2, axis=2), 2, axis=3)
+        assert not np.any(B[~at_max])            # nothing lands on an element that is not a maximum
+        del B, If, at_max
 
 
 def test_config5_pool_sampled(ng):
@@ -134,7 +140,9 @@ def test_config5_pool_sampled(ng):
         ng.fprop_pool(layer, dI, dO)
         ng.bprop_pool(layer, dI, dE, dB)
         O = dO.get()
-        wins = [(int(rng.integers(256)), 0, int(rng.integers(27)), int(rng.integers(27))) for _ in range(64)]
+        wins = [(int(rng.integers(256)), 0, int(rng.integers(27)), int(rng.integers(27))) for _ in range(256)]
+        wins += [(int(rng.integers(256)), 0, e, int(rng.integers(27))) for e in (0, 26) for _ in range(8)]
+        wins += [(int(rng.integers(256)), 0, int(rng.integers(27)), e) for e in (0, 26) for _ in range(8)]
         wins += [(0, 0, 0, 0), (255, 0, 26, 26), (7, 0, 0, 26), (9, 0, 26, 0)]
         ref = orc.ref_pool_fprop_pixels(I, op, layer.JTRS, wins, layer.padding, layer.strides)
         got = np.stack([O[w] for w in wins])
