@@ -279,6 +279,30 @@ def test_batchnorm_expression(ng, shape):
     np.testing.assert_allclose(O32.get(), orc.ref_ew(st, shape), rtol=2e-5, atol=2e-5)
 
 
+def test_config5_batchnorm_full_shape(ng):
+    """(4096, 8192) fp16 rows, the benchmark's own shape: nearest rounding within
+    one ulp of the float64 closed form; the stochastic store bit-exact against the
+    numpy restatement fed the kernel's own fp32 values and the same stream"""
+    from nervanagpu_amd import NervanaGPU
+    shape = (4096, 8192)
+    a = np.random.default_rng(4).uniform(0, 1, shape).astype(np.float16)
+    A = ng.array(a)
+    A[:] = bn_expr(ng, A, 1e-3)
+    ref = orc.ref_batchnorm_rows(a, 1e-3)
+    assert_fp16_within_ulp(A.get(), ref, 1.0, "bn fp16 full shape", atol=1e-5)
+    assert np.abs(A.get().astype(np.float64).mean(axis=1)).max() < 2e-3      # rows end up centred
+
+    ngs = NervanaGPU(stochastic_round=True, seed=4)
+    S = ngs.array(a)
+    assert S.rounding == 10
+    P = ngs.empty(shape, dtype=np.float32)
+    P.rounding = 0
+    P[:] = bn_expr(ngs, S, 1e-3)
+    S[:] = bn_expr(ngs, S, 1e-3)
+    r = orc.rand_sr16(4, ngs.rng_counter, np.arange(a.size, dtype=np.uint32)).reshape(shape)
+    assert np.array_equal(S.get().view(np.uint16), orc.round_stochastic_fp16(P.get(), 10, r).view(np.uint16))
+
+
 def test_stochastic_rounding_store_bit_exact(ng):
     """fp16 SR store: bit-exact against the numpy restatement fed the same stream"""
     from nervanagpu_amd import NervanaGPU
