@@ -76,6 +76,8 @@ extern "C" int ng_conv_update(const void* plan, int in_dtype, int out_dtype, con
         if (in_dtype == NG_F16 && out_dtype == NG_F16) return update_h<_Float16, _Float16>(*pl, I, E, gradF, alpha, workspace, workspace_bytes, st);
         if (in_dtype == NG_U8 && out_dtype == NG_F32)  return update_h<u8_t, float>(*pl, I, E, gradF, alpha, workspace, workspace_bytes, st);
         if (in_dtype == NG_U8 && out_dtype == NG_F16)  return update_h<u8_t, _Float16>(*pl, I, E, gradF, alpha, workspace, workspace_bytes, st);
+        if (in_dtype == NG_I8 && out_dtype == NG_F32)  return update_h<s8_t, float>(*pl, I, E, gradF, alpha, workspace, workspace_bytes, st);
+        if (in_dtype == NG_I8 && out_dtype == NG_F16)  return update_h<s8_t, _Float16>(*pl, I, E, gradF, alpha, workspace, workspace_bytes, st);
     } else if (in_dtype == NG_F32 && out_dtype == NG_F32) {
         if (pl->p.N % 16 == 0)
             return launch_update<float, float, float, true, 128, 128, 16, 2, 2>(*pl, I, E, gradF, alpha, workspace, workspace_bytes, st);

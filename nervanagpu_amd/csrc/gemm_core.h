@@ -989,10 +989,16 @@ struct ScaleStoreEpilogue {
         if (vec && beta == 0.0f && sr_bits == 0) {
             // common case, kept free of the rounding-stream arithmetic:
             // scale, optional relu, nearest rounding, 16-byte stores
-            const float lo = relu ? 0.0f : -3.402823466e+38f;
+            // (the clamp only exists with relu: NaN and infinities of an
+            // unrectified product must reach the output)
             bits_t out[8];
+            if (relu) {
 #pragma unroll
-            for (int e = 0; e < 8; e++) out[e] = StoreBits<T>::round(fmaxf(acc[e] * alpha, lo), 0, 0, 0, 0);
+                for (int e = 0; e < 8; e++) out[e] = StoreBits<T>::round(fmaxf(acc[e] * alpha, 0.0f), 0, 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) out[e] = StoreBits<T>::round(acc[e] * alpha, 0, 0, 0, 0);
+            }
             if (mask) mask8(out, offset);
 #pragma unroll
             for (int q = 0; q < NV; q++)

@@ -205,9 +205,13 @@ void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char
             // Branch-free, in the element type: the running maximum over all taps
             // (two fp16 elements per instruction), then a scan from the last tap
             // to the first for the first one that holds it: the element the
-            // reference's strict '>' scan keeps.  Taps outside the image become -inf.
+            // reference's strict '>' scan keeps.  That scan starts from -FLT_MAX at
+            // slot 0 (kernels/sass/hpool_max.sass:218-219), so taps outside the image
+            // count as -FLT_MAX (-inf once narrowed to fp16), a window without any
+            // tap inside the image yields that value, and a window in which nothing
+            // exceeds it keeps slot 0: the same results as the generic loop below.
             typedef typename Lanes<T, VEC>::type lanes_t;
-            const T lowest = (T)(-__builtin_huge_valf());
+            const T lowest = (T)(-NG_FLT_MAX);
             lanes_t taps[NTAP];
             bool all_ok = true;
 #pragma unroll
@@ -220,7 +224,7 @@ void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char
                 for (int tap = 0; tap < NTAP; tap++)
                     if (!ok[tap]) taps[tap] = Lanes<T, VEC>::splat(lowest);
             }
-            lanes_t top = taps[0];
+            lanes_t top = Lanes<T, VEC>::max(Lanes<T, VEC>::splat(lowest), taps[0]);
 #pragma unroll
             for (int tap = 1; tap < NTAP; tap++) top = Lanes<T, VEC>::max(top, taps[tap]);
             const long o = ((long)k * per_map + inner) * VEC;
@@ -232,6 +236,10 @@ void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char
 #pragma unroll
                     for (int i = 0; i < VEC; i++)
                         slot_of[i] = (Lanes<T, VEC>::get(taps[tap], i) == Lanes<T, VEC>::get(top, i)) ? tap : slot_of[i];
+                }
+                if (!all_ok) {
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) slot_of[i] = (Lanes<T, VEC>::get(top, i) > lowest) ? slot_of[i] : 0;
                 }
                 if (g.relu_mask) {
 #pragma unroll

@@ -111,6 +111,11 @@ def test_conv_uint8_input_bit_exact(ng):
     ng.fprop_conv(layer, ng.array(Is8, dtype=np.int8), dF, O8)
     ng.fprop_conv(layer, ng.array(Is8.astype(np.float16)), dF, Oh)
     assert np.array_equal(O8.get().view(np.uint16), Oh.get().view(np.uint16))
+    ng.update_conv(layer, ng.array(Is8, dtype=np.int8), dE, U8)
+    ng.update_conv(layer, ng.array(Is8.astype(np.float16)), dE, Uh)
+    assert np.array_equal(U8.get(), Uh.get())
+    assert_fp32_close(U8.get(), orc.ref_conv_update(Is8.astype(np.float32), E, layer.dimF, layer.padding, layer.strides),
+                      1e-5, "i8 update")
 
 
 def test_conv_adjoint_identity_gpu(ng):
@@ -241,6 +246,38 @@ def test_config5_conv3d(ng):
         E = rng.uniform(-1, 1, layer.dimO).astype(np.float16)
         return I, F, E
     _sampled_layer_check(ng, layer, 4, gen, npix=256, nrows=4)
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("geom", [(10, 10, 3, 3, 0, 0, 2, 2), (9, 12, 5, 3, 2, 1, 2, 1), (7, 7, 2, 2, 0, 0, 2, 2)])
+def test_deconv_layer_ops(ng, dtype, geom):
+    """DeconvLayer (nervanagpu/layers.py:509-537) is a ConvLayer whose input extent
+    H,W is derived from the wanted P,Q; a deconvolution runs it backwards: its
+    forward pass is bprop_conv (K maps of PxQ -> C maps of HxW), its backward pass
+    fprop_conv, its weight gradient update_conv.  All three against the oracle."""
+    P, Q, R, S, pad_h, pad_w, str_h, str_w = geom
+    N, C, K = 16, 24, 32
+    layer = ng.deconv_layer(dtype, N, C, K, P, Q, R, S, 0, pad_h, pad_w, 1, str_h, str_w)
+    assert layer.MPQ == (1, P, Q)
+    assert layer.DHW == (1, (P - 1) * str_h - 2 * pad_h + R, (Q - 1) * str_w - 2 * pad_w + S)
+    assert layer.dimO == (K, 1, P, Q, N) and layer.dimF == (C, 1, R, S, K)
+    small, F, big = _data(layer, dtype, 41)       # dimI-shaped, filters, dimO-shaped
+    dF = ng.array(F, dtype=dtype)
+    # forward of the deconvolution: upsample the (K,P,Q) maps to (C,H,W)
+    up = ng.empty(layer.dimI, dtype=dtype)
+    up.fill(7)
+    ng.bprop_conv(layer, dF, ng.array(big, dtype=dtype), up)
+    _check(up.get(), orc.ref_conv_bprop(F, big, layer.dimI, layer.padding, layer.strides), dtype, "deconv forward",
+           K * R * S)
+    # backward of the deconvolution: gradient w.r.t. the (K,P,Q) maps
+    down = ng.empty(layer.dimO, dtype=dtype)
+    ng.fprop_conv(layer, ng.array(small, dtype=dtype), dF, down)
+    _check(down.get(), orc.ref_conv_fprop(small, F, layer.padding, layer.strides), dtype, "deconv backward", C * R * S)
+    # weight gradient
+    dU = ng.empty(layer.dimF, dtype=np.float32)
+    ng.update_conv(layer, ng.array(small, dtype=dtype), ng.array(big, dtype=dtype), dU)
+    assert_fp32_close(dU.get(), orc.ref_conv_update(small, big, layer.dimF, layer.padding, layer.strides), 1e-5,
+                      "deconv update")
 
 
 def test_deconv_layer_and_errors(ng):

@@ -284,6 +284,146 @@ def test_stochastic_rounding_bit_exact(ng):
     assert np.all(np.abs(got - ref) <= 2.0 ** -7 * np.abs(ref) * 1.01 + 1e-5)   # within one unit at 7 bits
 
 
+def _dyadic(rng, shape, step=16):
+    """multiples of 1/step in [-1, 1]: products are multiples of 1/step^2, and
+    sums of up to 2^14 of them are exact in fp32 in any order"""
+    return (rng.integers(-step, step + 1, shape) / float(step)).astype(np.float16)
+
+
+def _fc_problem(op, M, K, N=128):
+    if op == "nn":
+        return M, N, K
+    if op == "tn":
+        return K, N, M
+    return M, K, N
+
+
+@pytest.mark.parametrize("MK", FC)
+@pytest.mark.parametrize("op", ["nn", "nt", "tn"])
+def test_config2_fc_shapes_stochastic_rounding_bit_exact(MK, op):
+    """The nine FC cases with stochastic-round outputs: contraction slices with
+    fp32 partial sums, the fixed-order reduce and its stochastic store (nn, tn),
+    and the one-launch store (nt), bit for bit against the numpy restatement of
+    fp32_to_fp16_rand (nervanagpu/float_ew.py:182-201) fed the same stream."""
+    from nervanagpu_amd import NervanaGPU
+    ngs = NervanaGPU(stochastic_round=10, seed=4321)
+    rng = np.random.default_rng(21)
+    m, n, k = _fc_problem(op, *MK)
+    A, B = _dyadic(rng, (m, k)), _dyadic(rng, (k, n))
+    dA = ngs.array(np.ascontiguousarray(A.T)).T if op[0] == "t" else ngs.array(A)
+    dB = ngs.array(np.ascontiguousarray(B.T)).T if op[1] == "t" else ngs.array(B)
+    for relu, beta in ((False, 0.0), (True, 0.5)):
+        C0 = (rng.integers(-64, 65, (m, n)) / 16.0).astype(np.float16)
+        C = ngs.array(C0)
+        ngs.dot(dA, dB, C, beta=beta, relu=relu)
+        pre = orc.ref_dot(A, B, C0, 1.0, beta, relu, acc_dtype=np.float32)     # exact
+        r = orc.rand_sr16(4321, ngs.rng_counter, np.arange(m * n, dtype=np.uint32)).reshape(m, n)
+        exp = orc.round_stochastic_fp16(pre, 10, r)
+        got = C.get()
+        assert np.array_equal(got.view(np.uint16), exp.view(np.uint16)), (op, MK, relu, beta)
+        assert not np.array_equal(got.view(np.uint16), pre.astype(np.float16).view(np.uint16))
+
+
+def test_config2_square_stochastic_rounding_bit_exact():
+    """4096^3 (256x256 tiles, one launch) with a stochastic store, with and without beta"""
+    from nervanagpu_amd import NervanaGPU
+    ngs = NervanaGPU(stochastic_round=10, seed=8)
+    rng = np.random.default_rng(22)
+    m = n = k = 4096
+    A, B = _dyadic(rng, (m, k)), _dyadic(rng, (k, n))
+    dA, dB = ngs.array(A), ngs.array(B)
+    for relu, beta in ((True, 0.0), (False, -0.5)):
+        C0 = (rng.integers(-64, 65, (m, n)) / 16.0).astype(np.float16)
+        C = ngs.array(C0)
+        ngs.dot(dA, dB, C, beta=beta, relu=relu)
+        pre = orc.ref_dot(A, B, C0, 1.0, beta, relu, acc_dtype=np.float32)
+        r = orc.rand_sr16(8, ngs.rng_counter, np.arange(m * n, dtype=np.uint32)).reshape(m, n)
+        assert np.array_equal(C.get().view(np.uint16), orc.round_stochastic_fp16(pre, 10, r).view(np.uint16)), (relu, beta)
+
+
+@pytest.mark.parametrize("shape", [(256, 128, 192), (130, 72, 64), (4096, 128, 1024)])
+def test_fp16_overflow_in_the_store(shape):
+    """|value| beyond the largest fp16: nearest rounding gives infinity,
+    stochastic rounding truncates to 65504 (round toward zero past the top,
+    nervanagpu/float_ew.py:182-201); exact operands, so the comparison is on bits.
+    Shapes: aligned one-launch store, ragged store, sliced contraction + reduce."""
+    from nervanagpu_amd import NervanaGPU
+    m, n, k = shape
+    rng = np.random.default_rng(23)
+    # integers -4..4 times powers of two chosen so that the sums have a spread of
+    # about 50000: every partial sum is an exact multiple of sa*sb below 2^24 units
+    e = int(round(np.log2(9821.0 / np.sqrt(k))))
+    sa, sb = 2.0 ** (e // 2), 2.0 ** (e - e // 2)
+    A = (rng.integers(-4, 5, (m, k)) * sa).astype(np.float16)
+    B = (rng.integers(-4, 5, (k, n)) * sb).astype(np.float16)
+    pre = orc.ref_dot(A, B, acc_dtype=np.float32)
+    assert (np.abs(pre) > 65504).mean() > 0.05 and (np.abs(pre) < 65504).mean() > 0.05
+    ngn = NervanaGPU(stochastic_round=False)
+    C = ngn.empty((m, n))
+    ngn.dot(ngn.array(A), ngn.array(B), C)
+    with np.errstate(over="ignore"):
+        exp = pre.astype(np.float16)
+    got = C.get()
+    assert np.isinf(exp).any()
+    assert np.array_equal(got.view(np.uint16), exp.view(np.uint16))
+    ngs = NervanaGPU(stochastic_round=10, seed=77)
+    C = ngs.empty((m, n))
+    ngs.dot(ngs.array(A), ngs.array(B), C)
+    r = orc.rand_sr16(77, ngs.rng_counter, np.arange(m * n, dtype=np.uint32)).reshape(m, n)
+    exp = orc.round_stochastic_fp16(pre, 10, r)
+    got = C.get()
+    assert np.array_equal(got.view(np.uint16), exp.view(np.uint16))
+    assert np.all(np.isfinite(got)) and (np.abs(got.astype(np.float32)) == 65504).any()
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("shape", [(128, 136, 64), (130, 67, 40)])
+def test_nan_and_infinities_reach_the_output(ng, dtype, shape):
+    """Without relu nothing clamps: a NaN or an infinity in A shows up in every
+    output of its row (aligned 16-byte stores and the ragged element-wise path);
+    with relu the reference's max(v, 0) turns NaN and -inf into 0."""
+    m, n, k = shape
+    rng = np.random.default_rng(24)
+    A = rng.uniform(0.5, 1, (m, k)).astype(dtype)
+    B = rng.uniform(0.5, 1, (k, n)).astype(dtype)
+    A[3, 5] = np.nan
+    A[7, 1] = np.inf
+    A[9, 2] = -np.inf
+    C = ng.empty((m, n), dtype=dtype)
+    ng.dot(ng.array(A, dtype=dtype), ng.array(B, dtype=dtype), C)
+    got = C.get()
+    assert np.all(np.isnan(got[3])) and np.all(got[7] == np.inf) and np.all(got[9] == -np.inf)
+    rest = np.ones(m, dtype=bool)
+    rest[[3, 7, 9]] = False
+    assert np.all(np.isfinite(got[rest]))
+    ng.dot(ng.array(A, dtype=dtype), ng.array(B, dtype=dtype), C, relu=True)
+    got = C.get()
+    assert np.all(got[3] == 0) and np.all(got[7] == np.inf) and np.all(got[9] == 0)
+
+
+def test_c_api_hgemm_colmajor(ng):
+    """nervana_hgemm_colmajor (kernels/C_interface/nervana_c_api.cu:402-420): the
+    column-major product is the row-major product of the swapped operands"""
+    from nervanagpu_amd import _lib
+    lib = _lib.load()
+    vp = ctypes.c_void_p
+    rng = np.random.default_rng(25)
+    m, n, k = 136, 72, 200
+    A = rng.uniform(-1, 1, (m, k)).astype(np.float16)
+    B = rng.uniform(-1, 1, (k, n)).astype(np.float16)
+    dA = ng.array(np.ascontiguousarray(A.T))       # column-major bytes of A(m,k)
+    dB = ng.array(np.ascontiguousarray(B.T))
+    dC = ng.empty((n, m), dtype=np.float16)        # column-major bytes of C(m,n)
+    assert lib.nervana_hgemm_colmajor(vp(dA.ptr), vp(dB.ptr), vp(dC.ptr), False, False, m, n, k,
+                                      m, k, m, 1.0, 0.0, None, False, True, None, -1)
+    assert_fp16_within_ulp(dC.get().T, orc.ref_dot(A, B, relu=True), 1.0, "hgemm colmajor", acc_atol(_absdot(A, B)))
+    # transposed A: stored (m,k) row-major = column-major (k,m), lda = k
+    dAt = ng.array(A)
+    assert lib.nervana_hgemm_colmajor(vp(dAt.ptr), vp(dB.ptr), vp(dC.ptr), True, False, m, n, k,
+                                      k, k, m, 1.0, 0.0, None, False, False, None, -1)
+    assert_fp16_within_ulp(dC.get().T, orc.ref_dot(A, B), 1.0, "hgemm colmajor tn", acc_atol(_absdot(A, B)))
+
+
 def test_error_paths(ng):
     A = ng.empty((8, 8), dtype=np.float16)
     B = ng.empty((8, 8), dtype=np.float32)

@@ -101,6 +101,38 @@ def test_max_pool_negative_inputs_padding_and_signed_zero_ties(ng, dtype):
                 np.testing.assert_allclose(dB.get(), refB, rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("geom", [(2, 2, 2, 2), (3, 3, 3, 2), (2, 3, 3, 1), (3, 3, 4, 3)])
+def test_max_pool_window_wholly_outside_the_image(ng, dtype, geom):
+    """A window that lies in the padding only: the reference's scan starts at
+    -FLT_MAX and finds nothing larger (kernels/sass/hpool_max.sass:218-219), so the
+    output is -FLT_MAX in fp32 and -inf once narrowed to fp16, on the compiled
+    2x2 / 3x3 window shapes and on the generic loop alike; the error of such a
+    window goes nowhere."""
+    R, S, pad, strd = geom
+    layer = ng.pool_layer(dtype, "max", 8, 3, 1, 7, 7, 1, 1, R, S, 0, 0, pad, pad, 1, 1, strd, strd)
+    rng = np.random.default_rng(13)
+    I = rng.uniform(-1, 1, layer.dimI).astype(dtype)
+    E = rng.uniform(0.5, 1, layer.dimO).astype(dtype)
+    dI, dE = ng.array(I, dtype=dtype), ng.array(E, dtype=dtype)
+    dO, dB = ng.empty(layer.dimO, dtype=dtype), ng.empty(layer.dimI, dtype=dtype)
+    ng.fprop_pool(layer, dI, dO)
+    ng.bprop_pool(layer, dI, dE, dB)
+    refO = orc.ref_pool_fprop(I, "max", layer.JTRS, layer.padding, layer.strides)
+    assert (refO == np.finfo(np.float32).min).any(), "geometry was meant to have windows in the padding only"
+    got = dO.get()
+    with np.errstate(over="ignore"):
+        exp = refO.astype(dtype)
+    assert np.array_equal(got, exp)
+    outside = refO == np.finfo(np.float32).min
+    assert np.all(got[outside] == (-np.inf if dtype == np.float16 else np.finfo(np.float32).min))
+    refB = orc.ref_pool_bprop(I, E, "max", layer.JTRS, layer.padding, layer.strides)
+    if dtype == np.float16:
+        assert_fp16_within_ulp(dB.get(), refB, 1.0, "max bprop", 1e-6)
+    else:
+        np.testing.assert_allclose(dB.get(), refB, rtol=1e-5, atol=1e-6)
+
+
 def test_config4_vgg_pool_shapes(ng):
     """2x2/2 max pooling at the five block ends of config 4, full shapes, every
     element: the forward result against a reshape + max, and the structure of
