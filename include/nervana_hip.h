@@ -101,6 +101,24 @@ int ng_gemm(int dtype, int trans_a, int trans_b, int m, int n, int k,
 size_t ng_gemm_workspace_bytes(int dtype, int trans_a, int trans_b, int m, int n, int k,
                                int batch_grid, int batch_loops);
 
+/* ng_gemm for callers that cannot allocate device memory or carry a workspace
+ * (code under stream capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.  Same arguments and results as
+ * ng_gemm given a workspace of ng_gemm_workspace_bytes(): the split partial
+ * sums go to a fixed array of NG_GEMM_STATIC_SCRATCH_BYTES that is part of the
+ * library image on every device (ng_init looks up its address).  A problem that
+ * wants more is refused with an error.  The call allocates and frees nothing.
+ * All calls on one device share the array: calls that overlap in time on one
+ * device (different streams or threads) race; calls on one stream do not. */
+#define NG_GEMM_STATIC_SCRATCH_BYTES (32u << 20)
+size_t ng_gemm_static_scratch_bytes(void);
+int ng_gemm_noalloc(int dtype, int trans_a, int trans_b, int m, int n, int k,
+                    const void* A, int lda, const void* B, int ldb, void* C, int ldc,
+                    float alpha, float beta, unsigned flags,
+                    unsigned seed, unsigned rng_stream,
+                    int batch_grid, long ldaz, long ldbz, long ldcz, int batch_loops,
+                    void* stream);
+
 /* GEMM-only C entry compatible with kernels/C_interface/nervana_c_api.h:31-128
  * (CUstream -> hipStream_t passed as void*; rand_state is unused because the
  * random stream is counter based; `grid` is accepted and ignored). */

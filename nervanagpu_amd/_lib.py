@@ -72,6 +72,11 @@ _SIGNATURES = {
                         c_int, c_long, c_long, c_long, c_int,
                         c_void_p, c_size_t, c_void_p]),
     "ng_gemm_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
+    "ng_gemm_static_scratch_bytes": (c_size_t, []),
+    "ng_gemm_noalloc": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int,
+                                c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
+                                c_float, c_float, c_uint, c_uint, c_uint,
+                                c_int, c_long, c_long, c_long, c_int, c_void_p]),
     "nervana_loadKernels": (c_bool, [c_char_p]),
     "nervana_unloadKernels": (c_bool, []),
     "nervana_randStateSizeBytes": (c_size_t, []),

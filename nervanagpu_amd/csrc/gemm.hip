@@ -5,6 +5,7 @@
 #include "gemm_core.h"
 
 #include <algorithm>
+#include <mutex>
 
 namespace ng {
 
@@ -196,6 +197,66 @@ int ng_gemm(int dtype, int trans_a, int trans_b, int m, int n, int k,
     if (m == 0 || n == 0) return 0;
     const unsigned sr_bits = sr_bits_of(flags, dtype);
     return dtype == NG_F16 ? dispatch<_Float16>(g, sr_bits) : dispatch<float>(g, sr_bits);
+}
+
+// ---- GEMM without allocation ------------------------------------------------
+// Split-contraction partial sums live in a device array that is part of the
+// loaded code object, so a caller that cannot allocate (stream capture, serving
+// loops) still gets the sliced schedule of the minibatch-wide shapes.  Every
+// device holds its own copy of the array; its address on a device is looked up
+// once, with that device current, and only that address is handed to kernels.
+}  // extern "C"
+
+static __device__ __align__(256) unsigned char scratch[NG_GEMM_STATIC_SCRATCH_BYTES];
+
+static constexpr int MAX_DEVICES = 64;
+static void* g_scratch_ptr[MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+namespace ng {
+
+// called by ng_init with `device` current; idempotent
+int gemm_static_scratch_setup(int device)
+{
+    if (device < 0 || device >= MAX_DEVICES) return fail(-30, "device index %d out of range", device);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[device]) return 0;
+    void* ptr = nullptr;
+    hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+    if (!ptr) return fail(-31, "static scratch has no device address");
+    g_scratch_ptr[device] = ptr;
+    return 0;
+}
+
+}  // namespace ng
+
+extern "C" {
+
+size_t ng_gemm_static_scratch_bytes(void) { return NG_GEMM_STATIC_SCRATCH_BYTES; }
+
+int ng_gemm_noalloc(int dtype, int trans_a, int trans_b, int m, int n, int k,
+                    const void* A, int lda, const void* B, int ldb, void* C, int ldc,
+                    float alpha, float beta, unsigned flags,
+                    unsigned seed, unsigned rng_stream,
+                    int batch_grid, long ldaz, long ldbz, long ldcz, int batch_loops,
+                    void* stream)
+{
+    int dev = -1;
+    NG_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES || !g_scratch_ptr[dev])
+        return fail(-32, "ng_gemm_noalloc: ng_init has not been called for device %d", dev);
+    if (m < 0 || n < 0 || k < 0 || batch_grid < 1 || batch_loops < 1)
+        return fail(-22, "ng_gemm_noalloc: bad extent");
+    const size_t need = ng_gemm_workspace_bytes(dtype, trans_a, trans_b, m, n, k, batch_grid, batch_loops);
+    if (need > (size_t)NG_GEMM_STATIC_SCRATCH_BYTES)
+        return fail(-33, "ng_gemm_noalloc: this problem wants %zu bytes of partial sums, the static scratch holds %zu; "
+                         "use ng_gemm with a caller workspace", need, (size_t)NG_GEMM_STATIC_SCRATCH_BYTES);
+    // partial slices are written in full by the split kernel before the reduce
+    // reads them, so nothing in the array has to start at zero
+    return ng_gemm(dtype, trans_a, trans_b, m, n, k, A, lda, B, ldb, C, ldc, alpha, beta, flags, seed, rng_stream,
+                   batch_grid, ldaz, ldbz, ldcz, batch_loops,
+                   need ? g_scratch_ptr[dev] : nullptr, need ? (size_t)NG_GEMM_STATIC_SCRATCH_BYTES : 0, stream);
 }
 
 // ---- GEMM-only C interface (kernels/C_interface/nervana_c_api.h) -----------

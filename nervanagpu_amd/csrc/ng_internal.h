@@ -14,6 +14,8 @@ namespace ng {
 int fail(int code, const char* fmt, ...);
 int hip_fail(hipError_t e, const char* what);
 int device_cu_count();
+// looks up this device's copy of the GEMM static scratch array (gemm.hip)
+int gemm_static_scratch_setup(int device);
 
 inline size_t dtype_size(int dtype)
 {

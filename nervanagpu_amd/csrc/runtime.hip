@@ -85,6 +85,8 @@ int ng_init(int device)
     NG_HIP(hipGetDeviceProperties(&g_prop, device));
     if (strncmp(g_prop.gcnArchName, "gfx950", 6) != 0)
         return fail(-3, "libnervana_hip is built for gfx950 only, device reports %s", g_prop.gcnArchName);
+    int rc = gemm_static_scratch_setup(device);
+    if (rc) return rc;
     g_device = device;
     return 0;
 }
