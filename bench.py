@@ -103,6 +103,29 @@ def time_gpu(ng, fn, iters=20, warmup=3):
     return end.time_since(start) / iters
 
 
+LLC_BYTES = 256e6            # Infinity Cache of the MI355X: buffers cycled through must exceed it
+COLD_BYTES = 640e6           # total footprint the rotating buffer sets of a "cold" row reach at least
+
+
+def cold_sets(set_bytes):
+    """number of buffer sets to rotate over so that a launch never finds its
+    operands in the last-level cache: at least 3 sets and COLD_BYTES in total"""
+    return int(max(3, -(-COLD_BYTES // max(set_bytes, 1))))
+
+
+def time_gpu_rotating(ng, fns, iters=20, warmup=3):
+    """like time_gpu, but launch k runs fns[k % len(fns)]: every fns[i] works on
+    its own buffers, so consecutive launches do not re-read cached operands"""
+    n = len(fns)
+    count = -(-iters // n) * n
+    state = {"i": 0}
+
+    def one():
+        fns[state["i"] % n]()
+        state["i"] += 1
+    return time_gpu(ng, one, count, max(warmup, n))
+
+
 def build_config2(ng):
     cases = []
     for (M, K) in FC_SHAPES:
@@ -177,23 +200,39 @@ VGG = [(3, 224, 64), (64, 224, 64), (64, 112, 128), (128, 112, 128), (128, 56, 2
        (256, 28, 512), (512, 28, 512), (512, 14, 512)]
 
 
-def row(name, ms, flops=None, nbytes=None, peak_tflops=PEAK_FP16_TFLOPS, cpu=None):
-    """cpu: (rate, unit, sample) of the numpy oracle on the host for the same case"""
-    r = {"case": name, "ms": ms}
+def row(name, ms, flops=None, nbytes=None, peak_tflops=PEAK_FP16_TFLOPS, cpu=None, cache="warm", ms_warm=None):
+    """One line of the per-case table.  `frac` is the fraction of the roofline that
+    bounds the case: min(matrix peak, arithmetic intensity x HBM peak) for the
+    contractions, HBM peak for pooling / elementwise.  cache: "cold" = timed over
+    rotating buffer sets larger than the last-level cache (then ms_warm is the
+    same case on one buffer set), "warm" = one buffer set re-used.
+    cpu: (rate, unit, sample) of the numpy oracle on the host for the same case"""
+    r = {"case": name, "ms": ms, "cache": cache}
+    if ms_warm is not None:
+        r["ms_warm"] = ms_warm
     if cpu:
         r["cpu_rate"], r["cpu_unit"], r["cpu_sample"] = cpu
     if flops:
         tf = flops / ms / 1e9
         r["tflops"] = tf
         r["pct_mfma_peak"] = 100.0 * tf / peak_tflops
+        ceiling = peak_tflops
         if nbytes:
             ceiling = min(peak_tflops, flops / nbytes * PEAK_HBM_GBS / 1e3)
             r["pct_of_min_roof"] = 100.0 * tf / ceiling
+        r["bound"] = "mfma" if ceiling >= peak_tflops else "hbm"
+        r["frac"] = tf / ceiling
     if nbytes:
         r["gbs"] = nbytes / ms / 1e6
         if not flops:
             r["pct_hbm_peak"] = 100.0 * r["gbs"] / PEAK_HBM_GBS
+            r["bound"] = "hbm"
+            r["frac"] = r["gbs"] / PEAK_HBM_GBS
     return r
+
+
+def hbm_bound(flops, nbytes, peak_tflops=PEAK_FP16_TFLOPS):
+    return flops / nbytes * PEAK_HBM_GBS / 1e3 < peak_tflops
 
 
 def conv_cpu(layer, rng):
@@ -222,25 +261,30 @@ def conv_rows(ng, tag, N, layers, rows, iters, cpu=False):
         else:
             C, HW, K = cfg
             layer = ng.conv_layer(np.float16, N, C, K, 1, HW, HW, 1, 3, 3, 0, 1, 1, 1, 1, 1)
-        I = ng.empty(layer.dimI)
-        F = ng.empty(layer.dimF)
-        E = ng.empty(layer.dimO)
-        O = ng.empty(layer.dimO)
-        B = ng.empty(layer.dimI)
-        U = ng.empty(layer.dimF, dtype=np.float32)
-        I[:] = ng.rand()
-        E[:] = ng.rand() - 0.5
-        F[:] = (ng.rand() - 0.5) * 0.05
         sI, sF, sO = layer.sizeI * 2, layer.sizeF * 2, layer.sizeO * 2
+        # layers priced by HBM (first layers, VGG conv1.2) are timed cold
+        cold = hbm_bound(layer.flops, sI + sF + sO)
+        nsets = cold_sets(sI + sO) if cold else 1
+        sets = []
+        for _ in range(nsets):
+            I, F, E = ng.empty(layer.dimI), ng.empty(layer.dimF), ng.empty(layer.dimO)
+            O, B, U = ng.empty(layer.dimO), ng.empty(layer.dimI), ng.empty(layer.dimF, dtype=np.float32)
+            I[:] = ng.rand()
+            E[:] = ng.rand() - 0.5
+            F[:] = (ng.rand() - 0.5) * 0.05
+            sets.append((I, F, E, O, B, U))
         nm = "%s C%d K%d %s %s" % (tag, layer.C, layer.K, layer.DHW, layer.TRS)
-        ms = time_gpu(ng, lambda: ng.fprop_conv(layer, I, F, O, relu=True), iters)
-        rows.append(row(nm + " fprop", ms, layer.flops, sI + sF + sO, cpu=conv_cpu(layer, rng) if cpu else None))
+        ops = [("fprop", lambda t: ng.fprop_conv(layer, t[0], t[1], t[3], relu=True), sI + sF + sO)]
         if tag != "conv3d":
-            ms = time_gpu(ng, lambda: ng.bprop_conv(layer, F, E, B), iters)
-            rows.append(row(nm + " bprop", ms, layer.flops, sI + sF + sO))
-            ms = time_gpu(ng, lambda: ng.update_conv(layer, I, E, U), iters)
-            rows.append(row(nm + " update", ms, layer.flops, sI + sO + layer.sizeF * 4))
-        del I, F, E, O, B, U
+            ops.append(("bprop", lambda t: ng.bprop_conv(layer, t[1], t[2], t[4]), sI + sF + sO))
+            ops.append(("update", lambda t: ng.update_conv(layer, t[0], t[2], t[5]), sI + sO + layer.sizeF * 4))
+        for opname, fn, nbytes in ops:
+            warm = time_gpu(ng, lambda: fn(sets[0]), iters)
+            ms = time_gpu_rotating(ng, [(lambda t=t: fn(t)) for t in sets], iters) if cold else warm
+            rows.append(row("%s %s" % (nm, opname), ms, layer.flops, nbytes, cache="cold" if cold else "warm",
+                            ms_warm=warm if cold else None,
+                            cpu=conv_cpu(layer, rng) if (cpu and opname == "fprop") else None))
+        del sets
 
 
 def pool_cpu(layer, nbytes):
@@ -260,22 +304,38 @@ def pool_cpu(layer, nbytes):
 
 def pool_rows(ng, tag, N, C, HW, win, strd, op, rows, iters, cpu=False):
     layer = ng.pool_layer(np.float16, op, N, C, 1, HW, HW, 1, 1, win, win, 0, 0, 0, 0, 1, 1, strd, strd)
-    I = ng.empty(layer.dimI)
-    E = ng.empty(layer.dimO)
-    O = ng.empty(layer.dimO)
-    B = ng.empty(layer.dimI)
-    I[:] = ng.rand()
-    E[:] = ng.rand()
     sI, sO = layer.sizeI * 2, layer.sizeO * 2
+    sets = []
+    for _ in range(cold_sets(2 * sI + 2 * sO)):
+        I, E, O, B = ng.empty(layer.dimI), ng.empty(layer.dimO), ng.empty(layer.dimO), ng.empty(layer.dimI)
+        I[:] = ng.rand()
+        E[:] = ng.rand()
+        sets.append((I, E, O, B))
     nm = "%s %s %dx%d/%d C%d %dx%d N%d" % (tag, op, win, win, strd, C, HW, HW, N)
-    ms = time_gpu(ng, lambda: ng.fprop_pool(layer, I, O), iters)
-    rows.append(row(nm + " fprop", ms, None, sI + sO, cpu=pool_cpu(layer, sI + sO) if cpu else None))
-    ms = time_gpu(ng, lambda: ng.bprop_pool(layer, I, E, B), iters)
-    rows.append(row(nm + " bprop", ms, None, (2 * sI + sO) if op == "max" else (sI + sO)))
+    warm = time_gpu(ng, lambda: ng.fprop_pool(layer, sets[0][0], sets[0][2]), iters)
+    ms = time_gpu_rotating(ng, [(lambda t=t: ng.fprop_pool(layer, t[0], t[2])) for t in sets], iters)
+    rows.append(row(nm + " fprop", ms, None, sI + sO, cache="cold", ms_warm=warm,
+                    cpu=pool_cpu(layer, sI + sO) if cpu else None))
+    warm = time_gpu(ng, lambda: ng.bprop_pool(layer, sets[0][0], sets[0][1], sets[0][3]), iters)
+    ms = time_gpu_rotating(ng, [(lambda t=t: ng.bprop_pool(layer, t[0], t[1], t[3])) for t in sets], iters)
+    rows.append(row(nm + " bprop", ms, None, (2 * sI + sO) if op == "max" else (sI + sO), cache="cold", ms_warm=warm))
+
+
+def gemm_row(ng, prefix, c, iters, peak=PEAK_FP16_TFLOPS, cpu=None):
+    """GEMM shapes priced by HBM (minibatch-wide, batched) are timed cold: the
+    same product over rotating operand sets; matrix-bound shapes on one set"""
+    if not hbm_bound(c.flops, c.bytes, peak):
+        return row(prefix + c.name(), time_gpu(ng, c.run, iters), c.flops, c.bytes, peak, cpu=cpu)
+    clones = [c] + [GemmCase(ng, c.op, c.m, c.n, c.k, c.relu, c.sr, c.dtype, c.batch, seed=100 + i)
+                    for i in range(cold_sets(c.bytes) - 1)]
+    warm = time_gpu(ng, c.run, iters)
+    ms = time_gpu_rotating(ng, [x.run for x in clones], iters)
+    return row(prefix + c.name(), ms, c.flops, c.bytes, peak, cpu=cpu, cache="cold", ms_warm=warm)
 
 
 def all_cases(ng, cases, iters=10, cpu=False):
-    """cpu: also time the numpy oracle on the host for one case of every kind
+    """Every configured case of configs 1-5 with its own roofline fraction.
+    cpu: also time the numpy oracle on the host for one case of every kind
     (np.dot for the GEMMs, sampled pixels / windows for convolution and pooling
     forward, the whole array for the elementwise cases)"""
     from nervanagpu_amd import NervanaGPU
@@ -289,25 +349,30 @@ def all_cases(ng, cases, iters=10, cpu=False):
     # config 1
     for op in ("nn", "tn"):
         c = GemmCase(ng, op, 1024, 1024, 1024, dtype=np.float32, seed=0)
-        rows.append(row("cfg1 " + c.name(), time_gpu(ng, c.run, iters), c.flops, c.bytes, PEAK_FP32_TFLOPS, cpu=gemm_cpu(c)))
+        rows.append(gemm_row(ng, "cfg1 ", c, iters, PEAK_FP32_TFLOPS, gemm_cpu(c)))
     # config 2
     for c in cases:
         if c.relu or c.sr:
             continue
-        rows.append(row("cfg2 " + c.name(), time_gpu(ng, c.run, iters), c.flops, c.bytes, cpu=gemm_cpu(c)))
+        rows.append(gemm_row(ng, "cfg2 ", c, iters, cpu=gemm_cpu(c) if c.op == "nn" else None))
+    for op in ("nt", "tn"):
+        rows.append(gemm_row(ng, "cfg2 ", GemmCase(ng, op, 4096, 4096, 4096), iters))
     for c in cases:
         if c.sr and c.relu and c.op == "nn":
-            rows.append(row("cfg2 " + c.name(), time_gpu(ng, c.run, iters), c.flops, c.bytes))
+            rows.append(gemm_row(ng, "cfg2 ", c, iters))
     conv_rows(ng, "cfg3 alexnet", 128, ALEXNET, rows, iters, cpu)
     conv_rows(ng, "cfg4 vgg", 64, VGG, rows, iters, cpu)
     for (C, HW) in ((64, 224), (128, 112), (256, 56), (512, 28), (512, 14)):
-        pool_rows(ng, "cfg4", 64, C, HW, 2, 2, "max", rows, iters, cpu)
+        pool_rows(ng, "cfg4", 64, C, HW, 2, 2, "max", rows, iters, cpu and HW == 224)
     # config 5
     ngs = NervanaGPU(stochastic_round=True, seed=4)
-    A = ngs.empty((4096, 8192))
-    A[:] = ngs.rand()
+    nsets = cold_sets(2 * 4096 * 8192 * 2)
+    As = [ngs.empty((4096, 8192)) for _ in range(nsets)]
+    Bs = [ngs.empty((4096, 8192)) for _ in range(nsets)]
+    for A in As:
+        A[:] = ngs.rand()
 
-    def bn():
+    def bn(A):
         A[:] = (A - ngs.mean(A, axis=1)) / ngs.sqrt(ngs.var(A, axis=1) + 1e-3)
     hA = np.random.default_rng(4).uniform(0, 1, (4096, 8192)).astype(np.float16) if cpu else None
     bn_cpu = ew_cpu = None
@@ -317,10 +382,18 @@ def all_cases(ng, cases, iters=10, cpu=False):
         h32 = hA.astype(np.float32)
         sec = cpu_seconds(lambda: (h32 * h32 + h32).astype(np.float16), repeats=1)
         ew_cpu = (2 * hA.nbytes / sec / 1e9, "GB/s", "numpy, whole array")
-    rows.append(row("cfg5 batchnorm (4096,8192) fp16 SR", time_gpu(ngs, bn, iters), None, 2 * A.nbytes, cpu=bn_cpu))
-    Bt = ngs.empty((4096, 8192))
-    rows.append(row("cfg5 elementwise a*b+c (4096,8192) fp16",
-                    time_gpu(ngs, lambda: Bt._assign(A * A + A), iters), None, 2 * A.nbytes, cpu=ew_cpu))
+    nb = 2 * As[0].nbytes
+    rows.append(row("cfg5 batchnorm (4096,8192) fp16 SR", time_gpu_rotating(ngs, [(lambda A=A: bn(A)) for A in As], iters),
+                    None, nb, cpu=bn_cpu, cache="cold", ms_warm=time_gpu(ngs, lambda: bn(As[0]), iters)))
+    for B in Bs:
+        B.rounding = 0
+    rows.append(row("cfg5 batchnorm (4096,8192) fp16 nearest",
+                    time_gpu_rotating(ngs, [(lambda A=A, B=B: B._assign((A - ngs.mean(A, axis=1)) / ngs.sqrt(ngs.var(A, axis=1) + 1e-3)))
+                                            for A, B in zip(As, Bs)], iters), None, nb, cache="cold"))
+    rows.append(row("cfg5 elementwise a*a+a (4096,8192) fp16",
+                    time_gpu_rotating(ngs, [(lambda A=A, B=B: B._assign(A * A + A)) for A, B in zip(As, Bs)], iters),
+                    None, nb, cpu=ew_cpu, cache="cold", ms_warm=time_gpu(ngs, lambda: Bs[0]._assign(As[0] * As[0] + As[0]), iters)))
+    del As, Bs
     for op in ("max", "avg"):
         pool_rows(ng, "cfg5", 128, 256, 56, 3, 2, op, rows, iters, cpu)
     conv_rows(ng, "conv3d", 32, [(64, 16, 28, 28, 128, 3, 3, 3)], rows, iters, cpu)
@@ -328,11 +401,12 @@ def all_cases(ng, cases, iters=10, cpu=False):
 
 
 def format_rows(rows):
-    lines = ["| case | GPU ms | TFLOP/s | % MFMA peak | % of min(MFMA, AI*BW) | GB/s | % HBM peak | CPU oracle |",
-             "|---|---|---|---|---|---|---|---|"]
+    lines = ["| case | GPU ms | cache | ms warm | TFLOP/s | % MFMA peak | % of min(MFMA, AI*BW) | GB/s | % HBM peak | CPU oracle |",
+             "|---|---|---|---|---|---|---|---|---|---|"]
     for r in rows:
-        lines.append("| %s | %.4f | %s | %s | %s | %s | %s | %s |" % (
-            r["case"], r["ms"],
+        lines.append("| %s | %.4f | %s | %s | %s | %s | %s | %s | %s | %s |" % (
+            r["case"], r["ms"], r.get("cache", ""),
+            "%.4f" % r["ms_warm"] if "ms_warm" in r else "",
             "%.1f" % r["tflops"] if "tflops" in r else "",
             "%.1f" % r["pct_mfma_peak"] if "pct_mfma_peak" in r else "",
             "%.1f" % r["pct_of_min_roof"] if "pct_of_min_roof" in r else "",
@@ -342,10 +416,41 @@ def format_rows(rows):
     return "\n".join(lines)
 
 
-# HBM bytes per launch of the 4096^3 kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on
-# `bench.py --calibrate`, each scaled by the same counter's reading for the 256 MiB copy
-# (98530 KiB x 2.0 fetched + 32768 KiB x 1.0 written); algorithmic bytes are 100.7e6
-DOMINANT_TRAFFIC_BYTES = 235.3e6
+def compact(rows):
+    """the per-case rows as they go into the JSON line: short keys, rounded"""
+    out = []
+    for r in rows:
+        c = {"case": r["case"], "ms": round(r["ms"], 5), "cache": r["cache"], "bound": r["bound"], "frac": round(r["frac"], 4)}
+        if "ms_warm" in r:
+            c["ms_warm"] = round(r["ms_warm"], 5)
+        if "tflops" in r:
+            c["tflops"] = round(r["tflops"], 1)
+        else:
+            c["gbs"] = round(r["gbs"], 0)
+        if "cpu_rate" in r:
+            c["cpu"] = "%.3g %s (%s)" % (r["cpu_rate"], r["cpu_unit"], r["cpu_sample"])
+        out.append(c)
+    return out
+
+
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_4096_fp16_hbm_traffic.md")
+
+
+def dominant_traffic():
+    """HBM bytes per launch of the 4096^3 kernel as measured with rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE on `bench.py --calibrate` (each counter scaled by its
+    reading for the 256 MiB copy of the same run); the committed summary of that
+    measurement carries the figure on a line `traffic_bytes_per_launch: N`.
+    Counters cannot be read from inside this process, so the line is the source."""
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch:"):
+                    return float(line.split(":", 1)[1].split()[0])
+    except OSError:
+        pass
+    return None
+
 
 CAL_COPY_ELEMS = 1 << 27     # fp16 elements of the calibration copy: 256 MiB read + 256 MiB written
 
@@ -372,8 +477,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--all", action="store_true", help="also time every configured case")
-    ap.add_argument("--out", default=None, help="file for the --all table")
+    ap.add_argument("--all", action="store_true", help="print the per-case table (stderr, or --out FILE)")
+    ap.add_argument("--out", default=None, help="file for the per-case table")
+    ap.add_argument("--no-cases", action="store_true", help="only the headline step, no per-case rows")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calibrate", action="store_true",
                     help="only launch a plain copy of known size and the dominant GEMM a few times "
@@ -410,7 +516,9 @@ def main():
     achieved = dominant.flops / dom_ms / 1e9
     roofline = {"bound": "mfma", "kernel": "mfma_gemm_direct_kernel<fp16,256x256x64,A:KC,B:MC,2 stages> (4096^3 nn)",
                 "achieved": achieved, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                "frac": achieved / PEAK_FP16_TFLOPS, "traffic": DOMINANT_TRAFFIC_BYTES,
+                "frac": achieved / PEAK_FP16_TFLOPS, "traffic": dominant_traffic(),
+                "traffic_source": "profiles/gemm_4096_fp16_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; "
+                                  "not re-measured by this run)",
                 "launch_ms": dom_ms, "flops_per_launch": dominant.flops}
 
     result = {
@@ -429,15 +537,19 @@ def main():
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(cases)
 
-    if args.all:
+    if not args.no_cases:
+        # one row per kernel family and configured shape, timed in this same run:
+        # GEMM (configs 1, 2), convolution fprop/bprop/update (3, 4, 3-D), pooling,
+        # batch normalisation and elementwise (5); HBM-priced rows over rotating buffers
         rows = all_cases(ng, cases, cpu=not args.no_cpu)
-        table = format_rows(rows)
-        if args.out:
-            with open(args.out, "w") as f:
-                f.write(table + "\n")
-        else:
-            sys.stderr.write(table + "\n")
-        result["cases"] = rows
+        if args.all or args.out:
+            table = format_rows(rows)
+            if args.out:
+                with open(args.out, "w") as f:
+                    f.write(table + "\n")
+            else:
+                sys.stderr.write(table + "\n")
+        result["cases"] = compact(rows)
     print(json.dumps(result))
 
 
