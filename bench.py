@@ -455,21 +455,98 @@ def dominant_traffic():
 CAL_COPY_ELEMS = 1 << 27     # fp16 elements of the calibration copy: 256 MiB read + 256 MiB written
 
 
-def calibrate(ng):
-    """Counter calibration run: a flat copy kernel that reads and writes exactly
-    CAL_COPY_ELEMS * 2 bytes, then the 4096^3 fp16 GEMM, five launches each."""
+def profile_cases(ng):
+    """name -> (description, callable) of the single launches hardware counters are collected on"""
+    from nervanagpu_amd import NervanaGPU
+    out = {}
+
+    def gemm(op):
+        c = GemmCase(ng, op, 4096, 4096, 4096)
+        return (c.name(), c.run)
+    out["gemm"] = lambda: gemm("nn")
+    out["gemm_nt"] = lambda: gemm("nt")
+
+    def fc():
+        c = GemmCase(ng, "nn", 4096, 128, 9216)
+        return (c.name(), c.run)
+    out["fc"] = fc
+
+    def conv(C, HW, K, which):
+        layer = ng.conv_layer(np.float16, 64, C, K, 1, HW, HW, 1, 3, 3, 0, 1, 1, 1, 1, 1)
+        I, F, E = ng.empty(layer.dimI), ng.empty(layer.dimF), ng.empty(layer.dimO)
+        O, B, U = ng.empty(layer.dimO), ng.empty(layer.dimI), ng.empty(layer.dimF, dtype=np.float32)
+        I[:] = ng.rand()
+        E[:] = ng.rand() - 0.5
+        F[:] = (ng.rand() - 0.5) * 0.05
+        fn = {"fprop": lambda: ng.fprop_conv(layer, I, F, O, relu=True),
+              "bprop": lambda: ng.bprop_conv(layer, F, E, B),
+              "update": lambda: ng.update_conv(layer, I, E, U)}[which]
+        return ("vgg conv C%d K%d %dx%d N64 %s: I %d B, F %d B, O %d B" % (C, K, HW, HW, which, layer.sizeI * 2,
+                                                                          layer.sizeF * 2, layer.sizeO * 2), fn)
+    for which in ("fprop", "bprop", "update"):
+        out["conv64_" + which] = lambda which=which: conv(64, 224, 64, which)
+        out["conv512_" + which] = lambda which=which: conv(512, 28, 512, which)
+
+    def pool(which):
+        layer = ng.pool_layer(np.float16, "max", 128, 256, 1, 56, 56, 1, 1, 3, 3, 0, 0, 0, 0, 1, 1, 2, 2)
+        I, E, O, B = ng.empty(layer.dimI), ng.empty(layer.dimO), ng.empty(layer.dimO), ng.empty(layer.dimI)
+        I[:] = ng.rand()
+        E[:] = ng.rand()
+        fn = (lambda: ng.fprop_pool(layer, I, O)) if which == "fprop" else (lambda: ng.bprop_pool(layer, I, E, B))
+        return ("max pool 3x3/2 C256 56x56 N128 %s: I %d B, O %d B" % (which, layer.sizeI * 2, layer.sizeO * 2), fn)
+    out["pool_fprop"] = lambda: pool("fprop")
+    out["pool_bprop"] = lambda: pool("bprop")
+
+    def bn():
+        ngs = NervanaGPU(stochastic_round=True, seed=4)
+        A = ngs.empty((4096, 8192))
+        A[:] = ngs.rand()
+
+        def run():
+            A[:] = (A - ngs.mean(A, axis=1)) / ngs.sqrt(ngs.var(A, axis=1) + 1e-3)
+        return ("batch normalisation (4096,8192) fp16 in place, stochastic store: %d B read, %d B written" % (A.nbytes, A.nbytes), run)
+    out["bn"] = bn
+    return out
+
+
+def calibrate(ng, names):
+    """Counter collection run: a flat copy kernel that reads and writes exactly
+    CAL_COPY_ELEMS * 2 bytes, then each named case, five launches each."""
     from nervanagpu_amd import _lib
     src = ng.empty((CAL_COPY_ELEMS // 8192, 8192), dtype=np.float16)
     dst = ng.empty((CAL_COPY_ELEMS // 8192, 8192), dtype=np.float16)
     src.fill(1.0)
     for _ in range(5):
         dst._assign(src)
-    gemm = GemmCase(ng, "nn", 4096, 4096, 4096)
-    for _ in range(5):
-        gemm.run()
-    _lib.stream_sync(ng.stream)
+    table = profile_cases(ng)
+    done = {}
+    for name in names:
+        if name not in table:
+            sys.exit("bench.py --calibrate: unknown case %r (known: %s)" % (name, ", ".join(sorted(table))))
+        desc, fn = table[name]()
+        for _ in range(5):
+            fn()
+        _lib.stream_sync(ng.stream)
+        done[name] = desc
     print(json.dumps({"calibrate": {"copy_bytes_read": CAL_COPY_ELEMS * 2, "copy_bytes_written": CAL_COPY_ELEMS * 2,
-                                    "gemm": gemm.name()}}))
+                                    "cases": done}}))
+
+
+def mfma_ceiling(ng):
+    """The loop of back-to-back MFMAs without memory traffic (ng_probe_mfma_loop),
+    two workgroups of four wavefronts per CU, on constant and on random operands:
+    what the matrix pipes deliver at the clock the power limit allows."""
+    import ctypes
+    from nervanagpu_amd import _lib
+    blocks, out = 512, {}
+    buf = ng.empty((blocks, 256), dtype=np.float32)
+    for label, rnd in (("constant", 0), ("random", 1)):
+        for iters in (4000, 40000):
+            def run():
+                _lib.call("ng_probe_mfma_loop", blocks, iters, rnd, ctypes.c_void_p(buf.ptr), ng.stream)
+            ms = time_gpu(ng, run, iters=5, warmup=1)
+            out["%s operands, %d rounds (%.2f ms)" % (label, iters, ms)] = blocks * 4 * iters * 16 * 32768.0 / ms / 1e9
+    print(json.dumps({"mfma_ceiling_tflops": out, "peak": PEAK_FP16_TFLOPS}))
 
 
 def main():
@@ -481,9 +558,11 @@ def main():
     ap.add_argument("--out", default=None, help="file for the per-case table")
     ap.add_argument("--no-cases", action="store_true", help="only the headline step, no per-case rows")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--calibrate", action="store_true",
-                    help="only launch a plain copy of known size and the dominant GEMM a few times "
-                         "(the run hardware counters are collected on)")
+    ap.add_argument("--calibrate", nargs="?", const="gemm", default=None, metavar="CASES",
+                    help="only launch a plain copy of known size and the named cases (comma separated; "
+                         "default the dominant GEMM) five times each: the run hardware counters are collected on")
+    ap.add_argument("--mfma-ceiling", action="store_true",
+                    help="only time the MFMA loop without memory traffic (practical matrix-pipe ceiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (got --gpus %d); "
@@ -492,7 +571,10 @@ def main():
     from nervanagpu_amd import NervanaGPU, _lib
     ng = NervanaGPU(stochastic_round=False, bench=False, seed=1)
     if args.calibrate:
-        calibrate(ng)
+        calibrate(ng, [n for n in args.calibrate.split(",") if n])
+        return
+    if args.mfma_ceiling:
+        mfma_ceiling(ng)
         return
     cases = build_config2(ng)
     step_flops = sum(c.flops for c in cases)

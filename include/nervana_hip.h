@@ -225,6 +225,14 @@ int ng_dimshuffle(int dtype, const void* in, void* out, int C, int TRS, int K, v
 /* dst (dtype, nearest rounding) = src (fp32) */
 int ng_fp32_convert(int dtype, const float* src, void* dst, size_t count, void* stream);
 
+/* ---- measurement probe ----------------------------------------------------------
+ * No counterpart in the reference.  `blocks` workgroups of 256 threads run
+ * `iters` rounds of 16 independent v_mfma_f32_32x32x16_f16 per wavefront with no
+ * memory traffic (constant or pseudo-random operands) and write one float per
+ * thread to `out` (blocks * 256 floats).  Flops per launch:
+ * blocks * 4 * iters * 16 * 32768.  bench.py --mfma-ceiling times it. */
+int ng_probe_mfma_loop(int blocks, int iters, int random_data, float* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

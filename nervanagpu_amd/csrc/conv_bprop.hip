@@ -73,7 +73,8 @@ static int bprop_merged(const ConvPlan& pl, const T* Fm, const void* E, void* gr
     DenseLoader<T, MC, true> al{Fm, 0, pl.m_rpad, pl.m_rpad, J};
     const int nblk = BLOCKED ? p.K / BK : 1;
     GatherColsLoader<T, T, BLOCKED, BK> bl{(const T*)E, BLOCKED ? pl.d_merged_taps : pl.d_merged_flat, J, lat,
-                                           1, 1, 1, p.M, p.P, p.Q, MPQN, FastDiv::make((unsigned)nblk), nblk, p.K, 0};
+                                           1, 1, 1, p.M, p.P, p.Q, MPQN, FastDiv::make((unsigned)nblk), nblk, p.K, 0,
+                                           BLOCKED ? pl.m_taps : 0};
     MergedLatticeStoreEpilogue<T> epi{(T*)gradI, pl.m_rows, p.C, FastDiv::make((unsigned)p.C),
                                       FastDiv::make((unsigned)(p.str_h * p.str_w)), FastDiv::make((unsigned)p.str_w),
                                       (long)p.D * p.H * p.W * p.N, lat, p.str_d, p.str_h, p.str_w, p.D, p.H, p.W, alpha};
@@ -116,7 +117,7 @@ static int bprop_class(const ConvPlan& pl, const BpropClass& c, const void* F, c
                                            BLOCKED ? pl.d_bprop_taps + c.tap_offset : pl.d_bprop_flat + c.flat_offset,
                                            c.J, lat, 1, 1, 1, p.M, p.P, p.Q,
                                            MPQN, FastDiv::make((unsigned)(BLOCKED ? std::max(c.taps, 1) : nblk)), nblk, p.K,
-                                           BLOCKED ? c.taps : 0};
+                                           BLOCKED ? c.taps : 0, BLOCKED ? c.taps : 0};
     const int k_tiles = cdiv(c.J, BK);
     const bool dense = (p.str_d == 1 && p.str_h == 1 && p.str_w == 1);
     ScaleStoreEpilogue<T> depi{(T*)gradI, 0, ncols, p.C, ncols, alpha, 0.0f, 0u, 0u, 0u, 0u, 1u, (const T*)mask};

@@ -2,9 +2,11 @@
 // {h,s}conv_fprop_K64_N64 (nervanagpu/nervanagpu.py:642-650, 671-734).
 #include "conv_plan.h"
 
+#include <cstdlib>
+
 namespace ng {
 
-template <typename T, typename TIN, bool BLOCKED, int BM, int BN, int BK, int WM, int WN>
+template <typename T, typename TIN, bool BLOCKED, int BM, int BN, int BK, int WM, int WN, int NSTAGE = 2>
 static int fprop_tile(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags,
                       hipStream_t stream)
 {
@@ -19,14 +21,14 @@ static int fprop_tile(const ConvPlan& pl, const void* I, const void* F, void* O,
         FilterBlockLoader<T, BK> al{(const T*)F, p.K, pl.RST * p.K, FastDiv::make((unsigned)pl.RST), pl.RST, p.C};
         GatherColsLoader<T, TIN, true, BK> bl{(const TIN*)I, pl.d_fprop_taps, pl.CRST, lat,
                                               p.str_d, p.str_h, p.str_w, p.D, p.H, p.W,
-                                              DHWN, FastDiv::make((unsigned)pl.RST), nblk, p.C, pl.RST};
-        return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, epi, p.K, ncols, pl.RST * nblk, 1, stream, "conv fprop");
+                                              DHWN, FastDiv::make((unsigned)pl.RST), nblk, p.C, pl.RST, pl.RST};
+        return launch_core<T, BM, BN, BK, WM, WN, MC, MC, NSTAGE>(al, bl, epi, p.K, ncols, pl.RST * nblk, 1, stream, "conv fprop");
     } else {
         DenseLoader<T, MC, true> al{(const T*)F, 0, p.K, p.K, pl.CRST};
         GatherColsLoader<T, TIN, false, BK> bl{(const TIN*)I, pl.d_fprop_flat, pl.CRST, lat,
                                                p.str_d, p.str_h, p.str_w, p.D, p.H, p.W,
                                                0, FastDiv{0, 0}, 1, 0, 0};
-        return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, epi, p.K, ncols, cdiv(pl.CRST, BK), 1, stream, "conv fprop");
+        return launch_core<T, BM, BN, BK, WM, WN, MC, MC, NSTAGE>(al, bl, epi, p.K, ncols, cdiv(pl.CRST, BK), 1, stream, "conv fprop");
     }
 }
 
@@ -43,6 +45,15 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
         // by request latency, not by the matrix pipe: half-depth tiles halve the
         // LDS footprint, so twice as many workgroups per CU keep requests in flight
         if (!BLOCKED) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 32, 1, 4>(pl, I, F, O, alpha, flags, st);
+        if constexpr (BLOCKED && std::is_same<TIN, _Float16>::value) {
+            static const int exp = getenv("NG_EXP_FPROP") ? atoi(getenv("NG_EXP_FPROP")) : 0;
+            if (exp == 1) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 64, 1, 4, 3>(pl, I, F, O, alpha, flags, st);
+            if (exp == 2) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 32, 1, 4, 4>(pl, I, F, O, alpha, flags, st);
+            if (exp == 3) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 32, 1, 4, 3>(pl, I, F, O, alpha, flags, st);
+            if (exp == 4) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 32, 1, 4, 6>(pl, I, F, O, alpha, flags, st);
+            if (exp == 5) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 32, 1, 4, 2>(pl, I, F, O, alpha, flags, st);
+            if (exp == 6) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 64, 1, 4, 4>(pl, I, F, O, alpha, flags, st);
+        }
         return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 64, 1, 4>(pl, I, F, O, alpha, flags, st);
     }
 }

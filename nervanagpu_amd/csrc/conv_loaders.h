@@ -137,14 +137,31 @@ struct GatherColsLoader {
     // taps (tap-major re-fetched the data gradient's E of a 5x5 layer 8.7 times
     // from HBM).  The A operand's loader must use the same order.
     int             block_major_taps;
+    // BLOCKED: entries of `tab`.  A table of at most 64 taps is kept in registers,
+    // lane l holding entry l, and a tile fetches its tap with v_readlane: no memory
+    // access (and no wait for one) between the barrier of a tile step and its
+    // requests.  0 = not stated: tile() reads the table from memory.
+    int             ntaps = 0;
 
     // same-type inputs are plain 16-byte buffer loads (see DenseLoader::DIRECT)
     static constexpr bool DIRECT = std::is_same<T, TIN>::value;
-    static constexpr bool TILE_READS_TABLE = BLOCKED;
+    static constexpr bool TILE_READS_TABLE = false;
 
     struct Ctx { int base, z0, y0, x0, kr; };
     // k0: flat: first contraction row of the tile; BLOCKED: rows of the block that exist
     struct Tile { BufferRsrc rsrc; int toff, dz, dy, dx, k0; };
+    struct Wave { int off, dz, dy, dx; };
+
+    __device__ __forceinline__ bool lane_table() const { return ntaps > 0 && ntaps <= 64; }
+    __device__ __forceinline__ Wave wave_init(int lane) const
+    {
+        Wave w{0, 0, 0, 0};
+        if (BLOCKED && lane_table()) {
+            const TapEntry e = tab[min(lane, ntaps - 1)];
+            w.off = e.off; w.dz = e.dz; w.dy = e.dy; w.dx = e.dx;
+        }
+        return w;
+    }
 
     __device__ __forceinline__ Ctx prepare(int col, int kr) const
     {
@@ -159,7 +176,7 @@ struct GatherColsLoader {
         return c;
     }
 
-    __device__ __forceinline__ Tile tile(int kt, int k0, int /*zb*/) const
+    __device__ __forceinline__ Tile tile(int kt, int k0, int /*zb*/, const Wave& w) const
     {
         Tile t;
         t.rsrc = make_rsrc(X);
@@ -167,7 +184,13 @@ struct GatherColsLoader {
         if (BLOCKED) {
             int tap, blk;
             decode_tile(kt, blk_div, nblk, block_major_taps, tap, blk);
-            const TapEntry e = tab[tap];
+            TapEntry e;
+            if (lane_table()) {
+                e.off = __builtin_amdgcn_readlane(w.off, tap); e.dz = __builtin_amdgcn_readlane(w.dz, tap);
+                e.dy = __builtin_amdgcn_readlane(w.dy, tap);   e.dx = __builtin_amdgcn_readlane(w.dx, tap);
+            } else {
+                e = tab[tap];
+            }
             t.toff = e.off + blk * BK * row_stride;
             t.dz = e.dz; t.dy = e.dy; t.dx = e.dx;
             t.k0 = chan - blk * BK;
@@ -218,6 +241,8 @@ struct FilterBlockLoader {
 
     struct Ctx { unsigned off; int kr; };
     struct Tile { BufferRsrc rsrc; int rows; };
+    typedef NoWaveState Wave;
+    __device__ __forceinline__ Wave wave_init(int /*lane*/) const { return Wave{}; }
 
     __device__ __forceinline__ Ctx prepare(int m, int kr) const
     {
@@ -226,7 +251,7 @@ struct FilterBlockLoader {
         c.kr = kr;
         return c;
     }
-    __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/) const
+    __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/, const Wave&) const
     {
         const int blk = (int)tap_div.div((unsigned)kt);
         const int tap = kt - blk * ntaps;
@@ -259,10 +284,18 @@ struct FilterRowsLoader {
     int        ntaps;
 
     static constexpr bool DIRECT = true;
-    static constexpr bool TILE_READS_TABLE = true;
+    static constexpr bool TILE_READS_TABLE = false;
 
     struct Ctx { unsigned off; int kc; };
     struct Tile { BufferRsrc rsrc; int kvalid; };
+    // the filter positions of up to 64 class taps, one per lane (see GatherColsLoader::ntaps)
+    struct Wave { int trs; };
+    __device__ __forceinline__ Wave wave_init(int lane) const
+    {
+        Wave w{0};
+        if (ntaps <= 64) w.trs = tap_trs[min(lane, max(ntaps, 1) - 1)];
+        return w;
+    }
 
     __device__ __forceinline__ Ctx prepare(int row, int kc) const
     {
@@ -271,13 +304,14 @@ struct FilterRowsLoader {
         c.off = (row < C) ? ((unsigned)row * (unsigned)RSTK + (unsigned)kc) * (unsigned)sizeof(T) : NG_OOB_OFFSET;
         return c;
     }
-    __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/) const
+    __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/, const Wave& w) const
     {
         const int blk = (int)tap_div.div((unsigned)kt);
         const int tap = kt - blk * ntaps;
         Tile t;
         // the table entry is wavefront-uniform; the descriptor must live in scalar registers
-        const int trs = __builtin_amdgcn_readfirstlane(tap_trs[tap]);
+        const int trs = (ntaps <= 64) ? __builtin_amdgcn_readlane(w.trs, tap)
+                                      : __builtin_amdgcn_readfirstlane(tap_trs[tap]);
         t.rsrc = make_rsrc(F + (long)trs * K + (long)blk * BK);
         t.kvalid = K - blk * BK;
         return t;
@@ -310,6 +344,8 @@ struct GatherRowsLoader {
 
     struct Ctx { int off, dz, dy, dx, kc; };
     struct Tile { BufferRsrc rsrc; int pixbase, z0, y0, x0, k0; };
+    typedef NoWaveState Wave;
+    __device__ __forceinline__ Wave wave_init(int /*lane*/) const { return Wave{}; }
 
     __device__ __forceinline__ Ctx prepare(int r, int kc) const
     {
@@ -324,7 +360,7 @@ struct GatherRowsLoader {
         return c;
     }
 
-    __device__ __forceinline__ Tile tile(int kt, int k0, int /*zb*/) const
+    __device__ __forceinline__ Tile tile(int kt, int k0, int /*zb*/, const Wave&) const
     {
         Tile t;
         t.rsrc = make_rsrc(X);

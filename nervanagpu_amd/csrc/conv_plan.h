@@ -108,7 +108,7 @@ inline int pick_row_tile(int rows, int ncols, int bn)
     return best;
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, class AL, class BL, class Epi>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, int NSTAGE = 2, class AL, class BL, class Epi>
 inline int launch_core(const AL& al, const BL& bl, const Epi& epi, int rows, int ncols, int k_tiles, int splits,
                        hipStream_t stream, const char* what)
 {
@@ -118,7 +118,7 @@ inline int launch_core(const AL& al, const BL& bl, const Epi& epi, int rows, int
     s.passes = 1; s.splits = splits;
     s.tiles_m = cdiv(rows, BM);
     s.tiles_n = cdiv(ncols, BN);
-    launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB>(dim3(grid_tiles(s.tiles_m * s.tiles_n, splits), grid_slices(s.tiles_m * s.tiles_n, splits), 1), stream, al, bl, epi, s);
+    launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB, NSTAGE>(dim3(grid_tiles(s.tiles_m * s.tiles_n, splits), grid_slices(s.tiles_m * s.tiles_n, splits), 1), stream, al, bl, epi, s);
     NG_CHECK_LAUNCH(what);
     return 0;
 }

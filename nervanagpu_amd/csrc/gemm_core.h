@@ -183,10 +183,17 @@ __device__ __forceinline__ uint4_t buffer_load_chunk(BufferRsrc rsrc, unsigned b
 //                            the next tile can be scheduled between the MFMAs of
 //                            the current one
 //
+//   Wave wave_init(lane)     once per thread: per-lane state a loader wants to keep
+//                            in registers for tile() (e.g. a small table held one
+//                            entry per lane and fetched with v_readlane); passed
+//                            back as the last argument of tile()
+//
 // Dense row-major operand.  KC: element (r,k) at base[r*ld + k]; MC: at base[k*ld + r].
 // VEC: the host guarantees 16-byte alignment of every chunk, that chunks do not
 // straddle the matrix edge and that the matrix spans less than 4 GiB; otherwise
 // elements are fetched one by one.
+struct NoWaveState {};
+
 template <typename T, int LAYOUT, bool VEC>
 struct DenseLoader {
     const T* base;
@@ -202,6 +209,8 @@ struct DenseLoader {
 
     struct Ctx { unsigned off; int k; int r; };
     struct Tile { BufferRsrc rsrc; const T* p; int krem; };
+    typedef NoWaveState Wave;
+    __device__ __forceinline__ Wave wave_init(int /*lane*/) const { return Wave{}; }
 
     __device__ __forceinline__ Ctx prepare(int r, int kc) const
     {
@@ -214,7 +223,7 @@ struct DenseLoader {
         return c;
     }
 
-    __device__ __forceinline__ Tile tile(int /*kt*/, int k0, int zb) const
+    __device__ __forceinline__ Tile tile(int /*kt*/, int k0, int zb, const Wave& = Wave{}) const
     {
         Tile t;
         t.p = base + (long)zb * ldz + (long)k0 * (LAYOUT == KC ? 1 : ld);
@@ -437,9 +446,11 @@ void mfma_gemm_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     constexpr int G_PER = (N_CHUNKS + G_PARTS - 1) / G_PARTS;
     typename ALoad::Tile g_ta;
     typename BLoad::Tile g_tb;
+    const typename ALoad::Wave a_wave = aload.wave_init(lane);
+    const typename BLoad::Wave b_wave = bload.wave_init(lane);
     auto gtile = [&]() {
-        g_ta = aload.tile(g_kt, g_kt * BK, z + g_pass);
-        g_tb = bload.tile(g_kt, g_kt * BK, z + g_pass);
+        g_ta = aload.tile(g_kt, g_kt * BK, z + g_pass, a_wave);
+        g_tb = bload.tile(g_kt, g_kt * BK, z + g_pass, b_wave);
         if (++g_kt == s.k_tiles) { g_kt = 0; g_pass++; }
     };
     auto gload_part = [&](int part) {
@@ -729,12 +740,17 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     // have no registers to spare, and not when a descriptor reads a table: a
     // scalar load in flight makes every later LDS wait a full wait
     // (scalar and LDS operations share one counter and return out of order).
-    constexpr bool PREP_AHEAD = NT <= 256 && !ALoad::TILE_READS_TABLE && !BLoad::TILE_READS_TABLE;
+#ifndef NG_EXP_PREP
+#define NG_EXP_PREP 0
+#endif
+    constexpr bool PREP_AHEAD = (NT <= 256 || NG_EXP_PREP) && !ALoad::TILE_READS_TABLE && !BLoad::TILE_READS_TABLE;
     int g_left = ntiles;
+    const typename ALoad::Wave a_wave = aload.wave_init(lane);
+    const typename BLoad::Wave b_wave = bload.wave_init(lane);
     auto gprep = [&]() {
         if (g_left > 0) {
-            g_ta = aload.tile(g_kt, g_kt * BK, z + g_pass);
-            g_tb = bload.tile(g_kt, g_kt * BK, z + g_pass);
+            g_ta = aload.tile(g_kt, g_kt * BK, z + g_pass, a_wave);
+            g_tb = bload.tile(g_kt, g_kt * BK, z + g_pass, b_wave);
             if (++g_kt == s.k_tiles) { g_kt = 0; g_pass++; }
             g_left--;
         }
