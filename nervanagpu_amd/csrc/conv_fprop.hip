@@ -2,8 +2,6 @@
 // {h,s}conv_fprop_K64_N64 (nervanagpu/nervanagpu.py:642-650, 671-734).
 #include "conv_plan.h"
 
-#include <cstdlib>
-
 namespace ng {
 
 template <typename T, typename TIN, bool BLOCKED, int BM, int BN, int BK, int WM, int WN, int NSTAGE = 2>
@@ -45,15 +43,6 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
         // by request latency, not by the matrix pipe: half-depth tiles halve the
         // LDS footprint, so twice as many workgroups per CU keep requests in flight
         if (!BLOCKED) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 32, 1, 4>(pl, I, F, O, alpha, flags, st);
-        if constexpr (BLOCKED && std::is_same<TIN, _Float16>::value) {
-            static const int exp = getenv("NG_EXP_FPROP") ? atoi(getenv("NG_EXP_FPROP")) : 0;
-            if (exp == 1) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 64, 1, 4, 3>(pl, I, F, O, alpha, flags, st);
-            if (exp == 2) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 32, 1, 4, 4>(pl, I, F, O, alpha, flags, st);
-            if (exp == 3) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 32, 1, 4, 3>(pl, I, F, O, alpha, flags, st);
-            if (exp == 4) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 32, 1, 4, 6>(pl, I, F, O, alpha, flags, st);
-            if (exp == 5) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 32, 1, 4, 2>(pl, I, F, O, alpha, flags, st);
-            if (exp == 6) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 64, 1, 4, 4>(pl, I, F, O, alpha, flags, st);
-        }
         return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 64, 1, 4>(pl, I, F, O, alpha, flags, st);
     }
 }

@@ -25,6 +25,8 @@
 #include "ng_internal.h"
 #include "ng_device_common.h"
 
+#include <type_traits>
+
 namespace ng {
 
 typedef _Float16 half8_t   __attribute__((ext_vector_type(8)));
@@ -194,6 +196,11 @@ __device__ __forceinline__ uint4_t buffer_load_chunk(BufferRsrc rsrc, unsigned b
 // elements are fetched one by one.
 struct NoWaveState {};
 
+// loaders that can step a tile descriptor to the next contraction tile declare
+// `static constexpr bool INCREMENTAL = true` and advance(Tile&, bk)
+template <class L, class = void> struct LoaderIncremental { static constexpr bool value = false; };
+template <class L> struct LoaderIncremental<L, std::enable_if_t<L::INCREMENTAL>> { static constexpr bool value = true; };
+
 template <typename T, int LAYOUT, bool VEC>
 struct DenseLoader {
     const T* base;
@@ -230,6 +237,16 @@ struct DenseLoader {
         t.rsrc = make_rsrc(t.p);
         t.krem = kdim - k0;
         return t;
+    }
+
+    // the descriptor of the next contraction tile of the same pass: a pointer
+    // bump instead of the 64-bit products of tile()
+    static constexpr bool INCREMENTAL = true;
+    __device__ __forceinline__ void advance(Tile& t, int bk) const
+    {
+        t.p += (LAYOUT == KC) ? (long)bk : (long)bk * ld;
+        t.rsrc = make_rsrc(t.p);
+        t.krem -= bk;
     }
 
     // rows past the matrix edge and contraction indices past kdim read as zero
@@ -740,18 +757,25 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     // have no registers to spare, and not when a descriptor reads a table: a
     // scalar load in flight makes every later LDS wait a full wait
     // (scalar and LDS operations share one counter and return out of order).
-#ifndef NG_EXP_PREP
-#define NG_EXP_PREP 0
-#endif
-    constexpr bool PREP_AHEAD = (NT <= 256 || NG_EXP_PREP) && !ALoad::TILE_READS_TABLE && !BLoad::TILE_READS_TABLE;
+    constexpr bool PREP_AHEAD = NT <= 256 && !ALoad::TILE_READS_TABLE && !BLoad::TILE_READS_TABLE;
     int g_left = ntiles;
     const typename ALoad::Wave a_wave = aload.wave_init(lane);
     const typename BLoad::Wave b_wave = bload.wave_init(lane);
+    bool g_fresh = true;    // the next descriptor starts a pass (or is the first of this workgroup)
     auto gprep = [&]() {
         if (g_left > 0) {
-            g_ta = aload.tile(g_kt, g_kt * BK, z + g_pass, a_wave);
-            g_tb = bload.tile(g_kt, g_kt * BK, z + g_pass, b_wave);
-            if (++g_kt == s.k_tiles) { g_kt = 0; g_pass++; }
+            if constexpr (LoaderIncremental<ALoad>::value) {
+                if (g_fresh) g_ta = aload.tile(g_kt, g_kt * BK, z + g_pass, a_wave); else aload.advance(g_ta, BK);
+            } else {
+                g_ta = aload.tile(g_kt, g_kt * BK, z + g_pass, a_wave);
+            }
+            if constexpr (LoaderIncremental<BLoad>::value) {
+                if (g_fresh) g_tb = bload.tile(g_kt, g_kt * BK, z + g_pass, b_wave); else bload.advance(g_tb, BK);
+            } else {
+                g_tb = bload.tile(g_kt, g_kt * BK, z + g_pass, b_wave);
+            }
+            g_fresh = false;
+            if (++g_kt == s.k_tiles) { g_kt = 0; g_pass++; g_fresh = true; }
             g_left--;
         }
     };
