@@ -27,7 +27,7 @@ What is different is the kernel shape, chosen for CDNA4:
     (seed, launch counter, logical element index), so results are reproducible.
 """
 import ctypes
-from ctypes import c_float, c_int, c_uint, c_void_p
+from ctypes import c_float, c_int, c_long, c_uint, c_void_p
 
 import numpy as np
 
@@ -101,26 +101,18 @@ _fast_dims_cache = {}
 
 
 def _get_fast_ew_dims(size):
-    """2-D view of a flat contiguous tensor (nervanagpu/float_ew.py:1037-1055);
-    kept for callers that size their launches with it (compensated_sum)."""
-    hit = _fast_dims_cache.get(size)
-    if hit:
-        return hit
-    ew_size = 256
-    while ew_size > 0:
-        if size % ew_size == 0:
-            break
-        ew_size -= 32
-    if ew_size == 0:
-        ew_size = 255
-        while ew_size > 0:
-            if size % ew_size == 0:
-                break
-            ew_size -= 1
-    shape = (size // ew_size, ew_size)
-    res = (shape, _contiguous_strides(shape))
-    _fast_dims_cache[size] = res
-    return res
+    """(shape, strides) of the 2-D view under which the reference runs a flat
+    contiguous tensor (nervanagpu/float_ew.py:1037-1055): rows of the widest
+    length that divides `size`, tried first among the multiples of 32 from 256
+    down, then among all lengths from 255 down (1 always divides).  This
+    generator runs flat expressions as a single row; the function remains for
+    callers that shape their own views the reference's way."""
+    if size not in _fast_dims_cache:
+        candidates = list(range(256, 0, -32)) + list(range(255, 0, -1))
+        width = next(w for w in candidates if size % w == 0)
+        shape = (size // width, width)
+        _fast_dims_cache[size] = (shape, _contiguous_strides(shape))
+    return _fast_dims_cache[size]
 
 
 # ---------------------------------------------------------------------------
@@ -1169,3 +1161,102 @@ def call_compound_kernel(backend, *args):
         bound = _bound_cache[sig] = _BoundLaunch(plan, func, arg_order)
     bound(backend, args)
     return args[0]
+
+
+# ---------------------------------------------------------------------------
+# Kahan-compensated accumulate: one kernel, three reads and two writes
+# ---------------------------------------------------------------------------
+
+_compensated_sum_cache = {}
+
+
+def compensated_sum_source(code, stochastic, name="compensated_sum"):
+    """HIP source of  y = add*add_scale - cmp*cmp_scale;  t = round(sum + y);
+    cmp = round_nearest((t - sum) - y);  sum = t   on 2-D strided tensors
+    (the arithmetic of nervanagpu/float_ew.py:1453-1475: every step in fp32, the
+    running sum rounded like its tensor, the error term always to nearest).
+    Contiguous tensors run as one row of 8-element vectors; element e = row *
+    cols + col draws word e of the random stream."""
+    ct = _ctype(code)
+    idx = "(unsigned)(i + v)"
+    src = [_lib.common_header_text(), ""]
+    src.append('extern "C" __global__ __launch_bounds__(256)')
+    src.append("void %s(%s* __restrict__ sum, %s* __restrict__ cmp, const %s* __restrict__ add," % (name, ct, ct, ct))
+    src.append("        float cmp_scale, float add_scale, long n, int cols, int vec,")
+    src.append("        long rs_sum, long cs_sum, long rs_cmp, long cs_cmp, long rs_add, long cs_add,")
+    src.append("        unsigned sr_bits, unsigned rng_seed, unsigned rng_stream)")
+    src.append("{")
+    src.append("    const long stride = (long)gridDim.x * 256 * 8;")
+    src.append("    for (long i = ((long)blockIdx.x * 256 + threadIdx.x) * 8; i < n; i += stride) {")
+    src.append("        %s s[8], c[8], a[8];" % ct)
+    src.append("        long os[8], oc[8];")
+    src.append("        if (vec) {")
+    src.append("            typedef %s vt_ __attribute__((ext_vector_type(8)));" % ct)
+    src.append("            *reinterpret_cast<vt_*>(s) = *reinterpret_cast<const vt_*>(sum + i);")
+    src.append("            *reinterpret_cast<vt_*>(c) = *reinterpret_cast<const vt_*>(cmp + i);")
+    src.append("            *reinterpret_cast<vt_*>(a) = *reinterpret_cast<const vt_*>(add + i);")
+    src.append("        } else {")
+    src.append('            _Pragma("unroll") for (int v = 0; v < 8; v++) {')
+    src.append("                const long e = (i + v < n) ? i + v : n - 1;")
+    src.append("                const long r = e / cols, q = e - r * cols;")
+    src.append("                os[v] = r * rs_sum + q * cs_sum; oc[v] = r * rs_cmp + q * cs_cmp;")
+    src.append("                s[v] = sum[os[v]]; c[v] = cmp[oc[v]]; a[v] = add[r * rs_add + q * cs_add];")
+    src.append("            }")
+    src.append("        }")
+    src.append('        _Pragma("unroll") for (int v = 0; v < 8; v++) {')
+    src.append("            const float s32 = (float)s[v];")
+    src.append("            const float y32 = (float)a[v] * add_scale - (float)c[v] * cmp_scale;")
+    src.append("            const %s t = %s;" % (ct, _gen_round(code, "(s32 + y32)", stochastic, idx)))
+    src.append("            c[v] = %s;" % _gen_round(code, "(((float)t - s32) - y32)", 0, idx))
+    src.append("            s[v] = t;")
+    src.append("        }")
+    src.append("        if (vec) {")
+    src.append("            typedef %s vt_ __attribute__((ext_vector_type(8)));" % ct)
+    src.append("            *reinterpret_cast<vt_*>(sum + i) = *reinterpret_cast<const vt_*>(s);")
+    src.append("            *reinterpret_cast<vt_*>(cmp + i) = *reinterpret_cast<const vt_*>(c);")
+    src.append("        } else {")
+    src.append('            _Pragma("unroll") for (int v = 0; v < 8; v++)')
+    src.append("                if (i + v < n) { sum[os[v]] = s[v]; cmp[oc[v]] = c[v]; }")
+    src.append("        }")
+    src.append("    }")
+    src.append("}")
+    return "\n".join(src)
+
+
+def call_compensated_sum(backend, sum_tensor, cmp_tensor, add_tensor, cmp_scale, add_scale):
+    """launch the fused accumulate on three tensors of one shape and dtype
+    (at most two dimensions unless all are contiguous)"""
+    code = sum_tensor.dtype.str[1:]
+    assert code in ("f2", "f4"), "compensated_sum works on fp16 or fp32 tensors"
+    assert sum_tensor.shape == cmp_tensor.shape == add_tensor.shape
+    tensors = (sum_tensor, cmp_tensor, add_tensor)
+    assert not any(t.take_array for t in tensors)
+    rounding = int(sum_tensor.rounding or 0)
+    sr_bits = max(1, min(rounding, 10 if code == "f2" else 15)) if rounding else 0
+    key = (code, bool(rounding))
+    fn = _compensated_sum_cache.get(key)
+    if fn is None:
+        name = "compensated_sum_%s_%s" % (code, "sr" if rounding else "rn")
+        fn = _lib.Module(compensated_sum_source(code, bool(rounding), name), name).get_function(name)
+        _compensated_sum_cache[key] = fn
+    n = sum_tensor.size
+    if n == 0:
+        return sum_tensor
+    es = sum_tensor.dtype.itemsize
+    flat = all(t.is_contiguous for t in tensors)
+    vec = int(flat and n % 8 == 0 and all(int(t.gpudata) % (8 * es) == 0 for t in tensors))
+    if flat:
+        cols, strides = n, [(0, 1)] * 3
+    else:
+        assert len(sum_tensor.shape) == 2, "strided operands of compensated_sum must be two-dimensional"
+        cols, strides = sum_tensor.shape[1], [tuple(t.strides) for t in tensors]
+    seed, stream_id = backend._next_rng_stream() if rounding else (0, 0)
+    cus = _lib.device_attr(0)
+    blocks = max(1, min((n + 2047) // 2048, cus * 8))
+    args = [c_void_p(int(sum_tensor.gpudata)), c_void_p(int(cmp_tensor.gpudata)), c_void_p(int(add_tensor.gpudata)),
+            c_float(cmp_scale), c_float(add_scale), c_long(n), c_int(cols), c_int(vec)]
+    for rs, cs in strides:
+        args += [c_long(rs), c_long(cs)]
+    args += [c_uint(sr_bits), c_uint(seed), c_uint(stream_id)]
+    fn.launch((blocks, 1, 1), (256, 1, 1), backend.stream, args)
+    return sum_tensor

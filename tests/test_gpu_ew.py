@@ -386,3 +386,41 @@ def test_compensated_sum(ng):
         ng.compensated_sum(S, Cm, ng.array(a), 1.0, 0.5)
         s, c = orc.ref_compensated_sum(s, c, a, 1.0, 0.5)
         assert np.array_equal(S.get(), s) and np.array_equal(Cm.get(), c)
+
+
+def test_compensated_sum_stochastic_and_strided():
+    """the fused accumulate with a stochastic store of the running sum (bit exact
+    against the numpy restatement on the same stream, one stream per call), fp32
+    storage, and strided 2-D views (scalar path)"""
+    from nervanagpu_amd import NervanaGPU
+    ngs = NervanaGPU(stochastic_round=10, seed=31)
+    rng = np.random.default_rng(9)
+    s = rng.uniform(-1, 1, (48, 264)).astype(np.float16)
+    c = np.zeros_like(s)
+    S, Cm = ngs.array(s), ngs.array(c)
+    for step in range(3):
+        a = rng.uniform(-0.01, 0.01, s.shape).astype(np.float16)
+        before = ngs.rng_counter
+        ngs.compensated_sum(S, Cm, ngs.array(a), 0.75, 1.5)
+        assert ngs.rng_counter == before + 1
+        r = orc.rand_sr16(31, ngs.rng_counter, np.arange(s.size, dtype=np.uint32)).reshape(s.shape)
+        s, c = orc.ref_compensated_sum(s, c, a, 0.75, 1.5, rounding=10, r=r)
+        assert np.array_equal(S.get().view(np.uint16), s.view(np.uint16)), step
+        assert np.array_equal(Cm.get().view(np.uint16), c.view(np.uint16)), step
+    # fp32 storage, nearest rounding, on column slices of wider tensors
+    ngn = NervanaGPU(stochastic_round=False)
+    s32 = rng.uniform(-1, 1, (33, 70)).astype(np.float32)
+    c32 = rng.uniform(-1e-6, 1e-6, (33, 70)).astype(np.float32)
+    a32 = rng.uniform(-1e-3, 1e-3, (33, 70)).astype(np.float32)
+    S32, C32, A32 = (ngn.array(x, dtype=np.float32) for x in (s32, c32, a32))
+    ngn.compensated_sum(S32[:, 3:61], C32[:, 3:61], A32[:, 3:61], 1.0, 2.0)
+    es, ec = orc.ref_compensated_sum(s32[:, 3:61], c32[:, 3:61], a32[:, 3:61], 1.0, 2.0, dtype=np.float32)
+    gs, gc = S32.get(), C32.get()
+    assert np.array_equal(gs[:, 3:61], es) and np.array_equal(gc[:, 3:61], ec)
+    assert np.array_equal(gs[:, :3], s32[:, :3]) and np.array_equal(gs[:, 61:], s32[:, 61:])
+    # the reset of the compensation after kahan_reset calls
+    C32.kahan_reset = 1
+    C32.kahan_count = 2
+    ngn.compensated_sum(S32, C32, A32)
+    es2, _ = orc.ref_compensated_sum(gs, gc, a32, 0.0, 1.0, dtype=np.float32)
+    assert np.array_equal(S32.get(), es2) and C32.kahan_count == 1
