@@ -205,9 +205,12 @@ struct GatherColsLoader {
     {
         constexpr int ES = ChunkFetch<T, TIN>::ES;
         if (BLOCKED) {
-            const bool ok = (unsigned)(c.z0 + t.dz) < (unsigned)lim_d && (unsigned)(c.y0 + t.dy) < (unsigned)lim_h &&
-                            (unsigned)(c.x0 + t.dx) < (unsigned)lim_w && c.kr < t.k0;
-            return ok ? (unsigned)(c.base + t.toff) * ES : NG_OOB_OFFSET;
+            // bitwise, not short-circuit: the four tests and the offset are computed
+            // unconditionally, so no execution-mask branches surround the request
+            const bool ok = ((unsigned)(c.z0 + t.dz) < (unsigned)lim_d) & ((unsigned)(c.y0 + t.dy) < (unsigned)lim_h) &
+                            ((unsigned)(c.x0 + t.dx) < (unsigned)lim_w) & (c.kr < t.k0);
+            const unsigned off = (unsigned)(c.base + t.toff) * ES;
+            return ok ? off : NG_OOB_OFFSET;
         } else {
             const int k = t.k0 + c.kr;
             const TapEntry e = tab[min(k, J - 1)];
@@ -384,9 +387,10 @@ struct GatherRowsLoader {
     {
         constexpr int ES = ChunkFetch<T, TIN>::ES;
         if (BLOCKED) {
-            const bool ok = (unsigned)(t.z0 + c.dz) < (unsigned)D && (unsigned)(t.y0 + c.dy) < (unsigned)H &&
-                            (unsigned)(t.x0 + c.dx) < (unsigned)W;
-            return ok ? (unsigned)(t.pixbase + c.off) * ES : NG_OOB_OFFSET;
+            const bool ok = ((unsigned)(t.z0 + c.dz) < (unsigned)D) & ((unsigned)(t.y0 + c.dy) < (unsigned)H) &
+                            ((unsigned)(t.x0 + c.dx) < (unsigned)W);
+            const unsigned off = (unsigned)(t.pixbase + c.off) * ES;
+            return ok ? off : NG_OOB_OFFSET;
         } else {
             const int kk = t.k0 + c.kc;
             const int kc2 = min(kk, kdim - 1);
