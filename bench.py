@@ -393,6 +393,11 @@ def all_cases(ng, cases, iters=10, cpu=False):
     rows.append(row("cfg5 elementwise a*a+a (4096,8192) fp16",
                     time_gpu_rotating(ngs, [(lambda A=A, B=B: B._assign(A * A + A)) for A, B in zip(As, Bs)], iters),
                     None, nb, cpu=ew_cpu, cache="cold", ms_warm=time_gpu(ngs, lambda: Bs[0]._assign(As[0] * As[0] + As[0]), iters)))
+    # yardstick for the bandwidth rows: a plain device-to-device copy of the same
+    # footprint (64 MiB in, 64 MiB out), through the same rotation
+    rows.append(row("cfg5 plain copy (4096,8192) fp16 [yardstick]",
+                    time_gpu_rotating(ngs, [(lambda A=A, B=B: B._assign(A)) for A, B in zip(As, Bs)], iters),
+                    None, nb, cache="cold", ms_warm=time_gpu(ngs, lambda: Bs[0]._assign(As[0]), iters)))
     del As, Bs
     for op in ("max", "avg"):
         pool_rows(ng, "cfg5", 128, 256, 56, 3, 2, op, rows, iters, cpu)
