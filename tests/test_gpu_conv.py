@@ -193,7 +193,7 @@ def _sampled_layer_check(ng, layer, seed, gen, npix=256, nrows=6, in_dtype=np.fl
     U = dU.get().reshape(crst, layer.K)
     rows = np.unique(np.concatenate([rng.integers(0, crst, nrows), [0, crst - 1]]))
     refu = orc.ref_conv_update_rows(If, E, layer.dimF, rows, layer.padding, layer.strides)
-    assert_fp32_close(U[rows], refu, 2e-5, "update %s" % layer)
+    assert_fp32_close(U[rows], refu, 1e-5, "update %s" % layer)
 
 
 def _alexnet_data(rng, layer):

@@ -123,9 +123,9 @@ def test_reductions_axis1_and_axis0(ng, dtype, shape):
         ng.mean(A, axis=axis, out=O)
         np.testing.assert_allclose(O.get(), a32.astype(np.float64).mean(axis=axis, keepdims=True), rtol=1e-5, atol=2e-6)
         ng.var(A, axis=axis, out=O)
-        np.testing.assert_allclose(O.get(), a32.astype(np.float64).var(axis=axis, keepdims=True), rtol=2e-5, atol=1e-6)
+        assert_fp32_close(O.get(), a32.astype(np.float64).var(axis=axis, keepdims=True), 1e-5, "var axis %d" % axis)
         ng.std(A, axis=axis, out=O)
-        np.testing.assert_allclose(O.get(), a32.astype(np.float64).std(axis=axis, keepdims=True), rtol=2e-5, atol=1e-6)
+        assert_fp32_close(O.get(), a32.astype(np.float64).std(axis=axis, keepdims=True), 1e-5, "std axis %d" % axis)
         Oi = ng.empty(oshape, dtype=np.int32)
         ng.argmax(A, axis=axis, out=Oi)
         assert np.array_equal(Oi.get(), np.expand_dims(np.argmax(a32, axis=axis), axis))
