@@ -346,9 +346,32 @@ struct GatherRowsLoader {
     static constexpr bool TILE_READS_TABLE = false;
 
     struct Ctx { int off, dz, dy, dx, kc; };
-    struct Tile { BufferRsrc rsrc; int pixbase, z0, y0, x0, k0; };
+    // BLOCKED: (m, p, q, nb) = output pixel and block inside it, kept so that the
+    // next tile is a counter step instead of three divisions
+    struct Tile { BufferRsrc rsrc; int pixbase, z0, y0, x0, k0; int m, p, q, nb; };
     typedef NoWaveState Wave;
     __device__ __forceinline__ Wave wave_init(int /*lane*/) const { return Wave{}; }
+
+    static constexpr bool INCREMENTAL = true;
+    __device__ __forceinline__ void place(Tile& t) const
+    {
+        t.z0 = t.m * str_d; t.y0 = t.p * str_h; t.x0 = t.q * str_w;
+        t.pixbase = ((t.z0 * H + t.y0) * W + t.x0) * N + t.nb * BK;
+    }
+    __device__ __forceinline__ void advance(Tile& t, int bk) const
+    {
+        t.k0 += bk;
+        if (BLOCKED) {
+            if (++t.nb == npt) {
+                t.nb = 0;
+                if (++t.q == Q) {
+                    t.q = 0;
+                    if (++t.p * Q == PQ) { t.p = 0; t.m++; }   // p reached P
+                }
+            }
+            place(t);
+        }
+    }
 
     __device__ __forceinline__ Ctx prepare(int r, int kc) const
     {
@@ -370,15 +393,15 @@ struct GatherRowsLoader {
         t.k0 = k0;
         if (BLOCKED) {
             const unsigned pix = npt_div.div((unsigned)kt);
-            const int nb = kt - (int)pix * npt;
+            t.nb = kt - (int)pix * npt;
             const unsigned m = pq_div.div(pix);
             const unsigned rem = pix - m * PQ;
             const unsigned p = q_div.div(rem);
-            const unsigned q = rem - p * Q;
-            t.z0 = (int)m * str_d; t.y0 = (int)p * str_h; t.x0 = (int)q * str_w;
-            t.pixbase = ((t.z0 * H + t.y0) * W + t.x0) * N + nb * BK;
+            t.m = (int)m; t.p = (int)p; t.q = (int)(rem - p * Q);
+            place(t);
         } else {
             t.z0 = t.y0 = t.x0 = t.pixbase = 0;
+            t.m = t.p = t.q = t.nb = 0;
         }
         return t;
     }
