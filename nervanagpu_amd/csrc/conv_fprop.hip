@@ -2,6 +2,8 @@
 // {h,s}conv_fprop_K64_N64 (nervanagpu/nervanagpu.py:642-650, 671-734).
 #include "conv_plan.h"
 
+#include <cstdlib>
+
 namespace ng {
 
 template <typename T, typename TIN, bool BLOCKED, int BM, int BN, int BK, int WM, int WN, int NSTAGE = 2>
@@ -30,9 +32,46 @@ static int fprop_tile(const ConvPlan& pl, const void* I, const void* F, void* O,
     }
 }
 
+// Filter rows of three taps on unit strides share their activation tile (see
+// GatherRowSegLoader): N = 64 images, so a 256-column tile is four output pixels
+// of one image row and the shared tile is six input pixels wide.
+static bool shares_taps(const ConvPlan& pl)
+{
+    const ng_conv_params& p = pl.p;
+    return p.S == 3 && p.N == 64 && p.Q % 4 == 0 && p.C % 32 == 0 &&
+           p.str_d == 1 && p.str_h == 1 && p.str_w == 1;
+}
+
+template <int BM, int WM, int WN>
+static int fprop_shared_taps(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags,
+                             hipStream_t stream)
+{
+    typedef _Float16 T;
+    constexpr int BK = 32, TAPS = 3, COLS = 64;
+    const ng_conv_params& p = pl.p;
+    const int ncols = p.M * p.P * p.Q * p.N;
+    const int TR = p.T * p.R, nblk = cdiv(p.C, BK);
+    ScaleStoreEpilogue<T> epi{(T*)O, 0, ncols, p.K, ncols, alpha, 0.0f, (flags & NG_FLAG_RELU) ? 1u : 0u, 0u, 0u, 0u, 1u};
+    FilterTapRowLoader<T, BK, TAPS> al{(const T*)F, p.K, pl.RST * p.K, FastDiv::make((unsigned)TR), TR, p.C};
+    GatherRowSegLoader<T, BK, TAPS, COLS> bl{(const T*)I, PixelLattice::make(p.N, ncols, p.Q, p.P * p.Q), p.D, p.H, p.W,
+                                             p.pad_d, p.pad_h, p.pad_w, p.D * p.H * p.W * p.N,
+                                             FastDiv::make((unsigned)TR), FastDiv::make((unsigned)p.R), TR, p.R, p.C};
+    return launch_core<T, BM, 256, BK, WM, WN, MC, MC>(al, bl, epi, p.K, ncols, TR * nblk, 1, stream, "conv fprop (shared taps)");
+}
+
 template <typename TIN, bool BLOCKED>
 static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags, hipStream_t st)
 {
+    if constexpr (BLOCKED && std::is_same<TIN, _Float16>::value) {
+        static const bool allow = !getenv("NG_NO_SHARED_TAPS");
+        if (allow && shares_taps(pl)) {
+            switch (pick_row_tile(pl.p.K, pl.p.M * pl.p.P * pl.p.Q * pl.p.N, 256)) {
+            case 256: return fprop_shared_taps<256, 2, 4>(pl, I, F, O, alpha, flags, st);
+            case 128: return fprop_shared_taps<128, 2, 4>(pl, I, F, O, alpha, flags, st);
+            default:  return fprop_shared_taps<64, 1, 4>(pl, I, F, O, alpha, flags, st);
+            }
+        }
+    }
     switch (pick_row_tile(pl.p.K, pl.p.M * pl.p.P * pl.p.Q * pl.p.N, 256)) {
     case 256: return fprop_tile<_Float16, TIN, BLOCKED, 256, 256, 64, 2, 4>(pl, I, F, O, alpha, flags, st);
     // 128 rows on eight wavefronts: mid-sized layers run about one workgroup per

@@ -270,6 +270,118 @@ struct FilterBlockLoader {
     __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const { return buffer_load_chunk(t.rsrc, offset(t, c)); }
 };
 
+// ---- forward convolution with the horizontal taps of a filter row sharing one
+// ---- activation tile (unit strides) ------------------------------------------------
+// A contraction tile is (channel block, t, r): its B tile holds, for BK channels,
+// the input row segment under the tile's PIX = BN / N consecutive output pixels,
+// PIX + S - 1 pixels wide, and tap s multiplies the window that starts s pixels
+// (N columns) into it.  The S taps of a filter row thus move the activations
+// from L2 to LDS once instead of S times; the A tile stacks the S filter slices
+// (tap-major, BK channels each).
+//
+// B operand.  Output pixels of a tile must lie in one image row (the host checks
+// Q % PIX == 0).  Column r of the tile is input pixel x = q0 - pad_w + r / N of
+// image n = r % N; x outside the image reads zero, whatever the tap.
+template <typename T, int BK, int TAPS_, int TAP_COLS_>
+struct GatherRowSegLoader {
+    static constexpr int TAPS = TAPS_, TAP_COLS = TAP_COLS_;
+    const T*     X;
+    PixelLattice lat;          // output pixels (M, P, Q) x N
+    int          D, H, W;
+    int          pad_d, pad_h, pad_w;
+    int          row_stride;   // elements between consecutive channels (D*H*W*N)
+    FastDiv      tr_div, r_div;
+    int          TR, R;        // filter rows (t, r) per channel block; R
+    int          chan;         // channels
+
+    static constexpr bool DIRECT = true;
+    static constexpr bool TILE_READS_TABLE = false;
+
+    struct Ctx { int base, z0, y0, kr; };
+    struct Tile { BufferRsrc rsrc; int toff, dz, dy, k0; };
+    typedef NoWaveState Wave;
+    __device__ __forceinline__ Wave wave_init(int /*lane*/) const { return Wave{}; }
+
+    __device__ __forceinline__ Ctx prepare_seg(int n0, int r, int kr) const
+    {
+        Ctx c;
+        c.kr = kr;
+        c.base = 0; c.z0 = c.y0 = NG_FAR;
+        if (n0 >= lat.ncols) return c;
+        int iz, iy, ix0, nn0;
+        lat.split(n0, iz, iy, ix0, nn0);
+        const int pix = r / TAP_COLS, nn = r - pix * TAP_COLS;
+        const int ix = ix0 + pix - pad_w;
+        if ((unsigned)ix >= (unsigned)W) return c;
+        c.z0 = iz; c.y0 = iy;
+        c.base = ((iz * H + iy) * W + ix) * lat.N + nn + kr * row_stride;
+        return c;
+    }
+    __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/, const Wave&) const
+    {
+        Tile t;
+        t.rsrc = make_rsrc(X);
+        const int blk = (int)tr_div.div((unsigned)kt);
+        const int tr = kt - blk * TR;
+        const int ft = (int)r_div.div((unsigned)tr);
+        const int fr = tr - ft * R;
+        t.dz = ft - pad_d; t.dy = fr - pad_h;
+        t.toff = (t.dz * H + t.dy) * W * lat.N + blk * BK * row_stride;
+        t.k0 = chan - blk * BK;
+        return t;
+    }
+    __device__ __forceinline__ unsigned offset(const Tile& t, const Ctx& c) const
+    {
+        const bool ok = ((unsigned)(c.z0 + t.dz) < (unsigned)D) & ((unsigned)(c.y0 + t.dy) < (unsigned)H) & (c.kr < t.k0);
+        const unsigned off = (unsigned)(c.base + t.toff) * (unsigned)sizeof(T);
+        return ok ? off : NG_OOB_OFFSET;
+    }
+    __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const { return buffer_load_chunk(t.rsrc, offset(t, c)); }
+};
+
+// A operand of the same kernel: line s * BK + c of tile (block, t, r) is filter
+// row (channel block*BK + c, t, r, s), K contiguous output maps each.
+template <typename T, int BK, int TAPS>
+struct FilterTapRowLoader {
+    const T* F;
+    int      K;
+    int      RSTK;       // elements between consecutive channels
+    FastDiv  tr_div;
+    int      TR;         // filter rows (t, r)
+    int      C;
+
+    static constexpr bool DIRECT = true;
+    static constexpr bool TILE_READS_TABLE = false;
+
+    struct Ctx { unsigned off; int c; };
+    struct Tile { BufferRsrc rsrc; int rows; };
+    typedef NoWaveState Wave;
+    __device__ __forceinline__ Wave wave_init(int /*lane*/) const { return Wave{}; }
+
+    __device__ __forceinline__ Ctx prepare(int m, int kr) const
+    {
+        Ctx c;
+        const int tap = kr / BK;
+        c.c = kr - tap * BK;
+        c.off = (m < K) ? (unsigned)(c.c * RSTK + tap * K + m) * (unsigned)sizeof(T) : NG_OOB_OFFSET;
+        return c;
+    }
+    __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/, const Wave&) const
+    {
+        const int blk = (int)tr_div.div((unsigned)kt);
+        const int tr = kt - blk * TR;
+        Tile t;
+        t.rsrc = make_rsrc(F + (long)blk * BK * RSTK + (long)tr * TAPS * K);
+        t.rows = C - blk * BK;
+        return t;
+    }
+    __device__ __forceinline__ unsigned offset(const Tile& t, const Ctx& c) const
+    {
+        return c.c < t.rows ? c.off : NG_OOB_OFFSET;
+    }
+    __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const { return buffer_load_chunk(t.rsrc, offset(t, c)); }
+};
+
 // A operand of the blocked data gradient: the filter F[c][trs][k] in place,
 // read as rows c with the contraction (tap, k): for one tap the k values of a
 // row are contiguous, so tile (tap, block) is a contraction-contiguous tile of

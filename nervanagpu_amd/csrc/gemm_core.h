@@ -196,6 +196,14 @@ __device__ __forceinline__ uint4_t buffer_load_chunk(BufferRsrc rsrc, unsigned b
 // elements are fetched one by one.
 struct NoWaveState {};
 
+// A B-operand loader may serve several horizontally adjacent filter taps from
+// ONE LDS tile: it then declares TAPS (> 1) and TAP_COLS, loads BN + (TAPS-1) *
+// TAP_COLS columns per tile through prepare_seg(), and tap s of the tile reads
+// its fragments TAP_COLS * s columns to the right.  The A tile of such a
+// kernel is TAPS * BK deep (tap-major).
+template <class L, class = void> struct LoaderTaps { static constexpr int taps = 1, cols = 0; };
+template <class L> struct LoaderTaps<L, std::enable_if_t<(L::TAPS > 1)>> { static constexpr int taps = L::TAPS, cols = L::TAP_COLS; };
+
 // loaders that can step a tile descriptor to the next contraction tile declare
 // `static constexpr bool INCREMENTAL = true` and advance(Tile&, bk)
 template <class L, class = void> struct LoaderIncremental { static constexpr bool value = false; };
@@ -695,8 +703,11 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     static_assert(NSTAGE >= 2, "need at least two LDS stages");
     constexpr int NT = WM * WN * 64;
     constexpr int KSTEP = Elem<T>::KSTEP;
-    using TA = SwizzledTile<T, LA, BM, BK>;
-    using TB = SwizzledTile<T, LB, BN, BK>;
+    constexpr int TAPS = LoaderTaps<BLoad>::taps;          // filter taps served by one B tile
+    constexpr int TAP_COLS = LoaderTaps<BLoad>::cols;      // columns by which a tap shifts its window
+    static_assert(TAPS == 1 || (LB == MC && TAP_COLS % 32 == 0), "shared taps need a row-contiguous B tile");
+    using TA = SwizzledTile<T, LA, BM, BK * TAPS>;
+    using TB = SwizzledTile<T, LB, BN + (TAPS - 1) * TAP_COLS, BK>;
     using FA = SwizzledFrag<LA, TA>;
     using FB = SwizzledFrag<LB, TB>;
     constexpr int CPT_A = TA::CHUNKS / NT;
@@ -736,7 +747,12 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
 #pragma unroll
     for (int i = 0; i < CPT_A; i++) { int r, k; TA::chunk_pos(tid + i * NT, r, k); actx[i] = aload.prepare(m0 + r, k); }
 #pragma unroll
-    for (int i = 0; i < CPT_B; i++) { int r, k; TB::chunk_pos(tid + i * NT, r, k); bctx[i] = bload.prepare(n0 + r, k); }
+    for (int i = 0; i < CPT_B; i++) {
+        int r, k;
+        TB::chunk_pos(tid + i * NT, r, k);
+        if constexpr (TAPS > 1) bctx[i] = bload.prepare_seg(n0, r, k);
+        else                    bctx[i] = bload.prepare(n0 + r, k);
+    }
 
     float16_t acc[TM][TN];
 #pragma unroll
@@ -748,7 +764,8 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
 
     int g_pass = t_begin / s.k_tiles;
     int g_kt = t_begin - g_pass * s.k_tiles;
-    constexpr int NSTEP = BK / KSTEP;
+    constexpr int KS = BK / KSTEP;              // k-steps per tap
+    constexpr int NSTEP = TAPS * KS;
     constexpr int N_CHUNKS = CPT_A + CPT_B;
     typename ALoad::Tile g_ta;
     typename BLoad::Tile g_tb;
@@ -794,19 +811,23 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     };
 
     // lane-constant fragment addresses
-    int fa_base[TM], fb_base[TN];
+    int fa_base[TM], fb_base[TAPS][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++) fa_base[i] = FA::base(wm * TM + i, lane);
 #pragma unroll
-    for (int j = 0; j < TN; j++) fb_base[j] = TA::BYTES + FB::base(wn * TN + j, lane);
+    for (int tap = 0; tap < TAPS; tap++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) fb_base[tap][j] = TA::BYTES + FB::base(wn * TN + j + tap * (TAP_COLS / 32), lane);
 
     Frag<T> fa[2][TM], fb[2][TN];
+    // k-step `step` of a tile: A lines 16*step .. +15; B lines 16*(step % KS) .. +15
+    // of the window of tap step / KS
     auto load_frags = [&](int stage_off, int step, Frag<T> (&a)[TM], Frag<T> (&b)[TN]) {
         const char* tile = smem + stage_off;
 #pragma unroll
         for (int i = 0; i < TM; i++) a[i] = FA::load(tile, fa_base[i], step);
 #pragma unroll
-        for (int j = 0; j < TN; j++) b[j] = FB::load(tile, fb_base[j], step);
+        for (int j = 0; j < TN; j++) b[j] = FB::load(tile, fb_base[step / KS][j], step % KS);
     };
     auto multiply = [&](const Frag<T> (&a)[TM], const Frag<T> (&b)[TN]) {
 #pragma unroll
@@ -879,7 +900,7 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
             for (int m = 0; m < N_MFMA; m++) {
                 mfma_step(ca[m / TN], cb[m % TN], acc[m / TN][m % TN]);
                 if (m < TM) na[m < TM ? m : 0] = FA::load(tile, fa_base[m < TM ? m : 0], 0);
-                else if (m < TM + TN) nb[m - TM < TN ? (m >= TM ? m - TM : 0) : 0] = FB::load(tile, fb_base[m - TM < TN ? (m >= TM ? m - TM : 0) : 0], 0);
+                else if (m < TM + TN) nb[m - TM < TN ? (m >= TM ? m - TM : 0) : 0] = FB::load(tile, fb_base[0][m - TM < TN ? (m >= TM ? m - TM : 0) : 0], 0);
 #pragma unroll
                 for (int q = 0; q < PER; q++) {
                     const int c = m * PER + q;

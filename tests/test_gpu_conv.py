@@ -30,6 +30,13 @@ SMALL = [
     (8, 16, 24, 1, 12, 9, 1, 7, 1, (0, 3, 0), (1, 1, 1)),
     (8, 8, 8, 6, 7, 7, 3, 3, 3, (1, 1, 1), (2, 2, 2)),
     (8, 8, 16, 1, 5, 5, 1, 5, 5, (0, 0, 0), (1, 1, 1)),
+    # 64 images, three taps per filter row, unit strides, output rows of a multiple of four pixels:
+    # forward runs with the taps of a filter row sharing one activation tile
+    (64, 32, 64, 1, 8, 8, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (64, 160, 72, 1, 5, 14, 1, 3, 3, (0, 0, 0), (1, 1, 1)),        # no padding, five channel blocks, ragged K
+    (64, 32, 32, 4, 6, 8, 2, 3, 3, (1, 1, 1), (1, 1, 1)),          # 3-D
+    (64, 64, 136, 1, 5, 8, 1, 1, 3, (0, 0, 1), (1, 1, 1)),         # one filter row
+    (64, 32, 16, 1, 4, 4, 1, 3, 3, (0, 1, 3), (1, 1, 1)),          # padding wider than the filter reach
 ]
 
 
