@@ -136,6 +136,35 @@ static int bprop_class(const ConvPlan& pl, const BpropClass& c, const void* F, c
     }
 }
 
+// Unit strides, filter rows of three taps, N = 64: the taps of a filter row share
+// one tile of E (see FilterTapColsLoader); a 256-column tile is four pixels of
+// one row of the input image.
+static bool shares_taps(const ConvPlan& pl)
+{
+    const ng_conv_params& p = pl.p;
+    return p.S == 3 && p.N == 64 && p.W % 4 == 0 && p.K % 32 == 0 &&
+           p.str_d == 1 && p.str_h == 1 && p.str_w == 1 && !pl.merged;
+}
+
+template <int BM, int WM, int WN>
+static int bprop_shared_taps(const ConvPlan& pl, const void* F, const void* E, void* gradI, float alpha,
+                             const void* mask, hipStream_t stream)
+{
+    typedef _Float16 T;
+    constexpr int BN = 256, BK = 32, TAPS = 3, COLS = 64;
+    const ng_conv_params& p = pl.p;
+    const int ncols = p.D * p.H * p.W * p.N;
+    const int TR = p.T * p.R, nblk = cdiv(p.K, BK);
+    ScaleStoreEpilogue<T> epi{(T*)gradI, 0, ncols, p.C, ncols, alpha, 0.0f, 0u, 0u, 0u, 0u, 1u, (const T*)mask};
+    FilterTapColsLoader<T, BK, TAPS> al{(const T*)F, p.C, p.K, pl.RST * p.K, FastDiv::make((unsigned)TR),
+                                        FastDiv::make((unsigned)p.R), TR, p.R};
+    GatherRowSegLoader<T, BK, TAPS, COLS> bl{(const T*)E, PixelLattice::make(p.N, ncols, p.W, p.H * p.W), p.M, p.P, p.Q,
+                                             p.T - 1 - p.pad_d, p.R - 1 - p.pad_h, p.S - 1 - p.pad_w,
+                                             p.M * p.P * p.Q * p.N,
+                                             FastDiv::make((unsigned)TR), FastDiv::make((unsigned)p.R), TR, p.R, p.K};
+    return launch_core<T, BM, BN, BK, WM, WN, KC, MC>(al, bl, epi, p.C, ncols, TR * nblk, 1, stream, "conv bprop (shared taps)");
+}
+
 template <bool BLOCKED>
 static int bprop_class_h(const ConvPlan& pl, const BpropClass& c, const void* F, const _Float16* Fs, const void* E,
                          void* gradI, float alpha, const void* mask, hipStream_t st)
@@ -168,6 +197,15 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
         hipLaunchKernelGGL(filter_relayout_kernel<T>, dim3(blocks), dim3(256), 0, stream,
                            (const T*)F, Fs, pl.d_tap_dest, p.C, pl.RST, p.K, pl.Kpad, pl.Cpad);
         NG_CHECK_LAUNCH("filter relayout");
+    }
+    if constexpr (sizeof(T) == 2) {
+        if (shares_taps(pl)) {
+            switch (pick_row_tile(p.C, p.D * p.H * p.W * p.N, 256)) {
+            case 256: return bprop_shared_taps<256, 2, 4>(pl, F, E, gradI, alpha, mask, stream);
+            case 128: return bprop_shared_taps<128, 2, 4>(pl, F, E, gradI, alpha, mask, stream);
+            default:  return bprop_shared_taps<64, 1, 4>(pl, F, E, gradI, alpha, mask, stream);
+            }
+        }
     }
     for (const BpropClass& c : pl.classes) {
         if (c.nz * c.ny * c.nx == 0) continue;

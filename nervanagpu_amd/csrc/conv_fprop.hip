@@ -2,8 +2,6 @@
 // {h,s}conv_fprop_K64_N64 (nervanagpu/nervanagpu.py:642-650, 671-734).
 #include "conv_plan.h"
 
-#include <cstdlib>
-
 namespace ng {
 
 template <typename T, typename TIN, bool BLOCKED, int BM, int BN, int BK, int WM, int WN, int NSTAGE = 2>
@@ -47,7 +45,7 @@ static int fprop_shared_taps(const ConvPlan& pl, const void* I, const void* F, v
                              hipStream_t stream)
 {
     typedef _Float16 T;
-    constexpr int BK = 32, TAPS = 3, COLS = 64;
+    constexpr int BN = 256, BK = 32, TAPS = 3, COLS = 64;
     const ng_conv_params& p = pl.p;
     const int ncols = p.M * p.P * p.Q * p.N;
     const int TR = p.T * p.R, nblk = cdiv(p.C, BK);
@@ -56,15 +54,14 @@ static int fprop_shared_taps(const ConvPlan& pl, const void* I, const void* F, v
     GatherRowSegLoader<T, BK, TAPS, COLS> bl{(const T*)I, PixelLattice::make(p.N, ncols, p.Q, p.P * p.Q), p.D, p.H, p.W,
                                              p.pad_d, p.pad_h, p.pad_w, p.D * p.H * p.W * p.N,
                                              FastDiv::make((unsigned)TR), FastDiv::make((unsigned)p.R), TR, p.R, p.C};
-    return launch_core<T, BM, 256, BK, WM, WN, MC, MC>(al, bl, epi, p.K, ncols, TR * nblk, 1, stream, "conv fprop (shared taps)");
+    return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, epi, p.K, ncols, TR * nblk, 1, stream, "conv fprop (shared taps)");
 }
 
 template <typename TIN, bool BLOCKED>
 static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags, hipStream_t st)
 {
     if constexpr (BLOCKED && std::is_same<TIN, _Float16>::value) {
-        static const bool allow = !getenv("NG_NO_SHARED_TAPS");
-        if (allow && shares_taps(pl)) {
+        if (shares_taps(pl)) {
             switch (pick_row_tile(pl.p.K, pl.p.M * pl.p.P * pl.p.Q * pl.p.N, 256)) {
             case 256: return fprop_shared_taps<256, 2, 4>(pl, I, F, O, alpha, flags, st);
             case 128: return fprop_shared_taps<128, 2, 4>(pl, I, F, O, alpha, flags, st);

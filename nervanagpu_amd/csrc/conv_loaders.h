@@ -382,6 +382,57 @@ struct FilterTapRowLoader {
     __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const { return buffer_load_chunk(t.rsrc, offset(t, c)); }
 };
 
+// A operand of the data gradient with shared taps: rows are channels c, the
+// contraction is (mirrored tap s', output map k) over BK output maps, k contiguous.
+// Tile (block, t', r') reads filter row (T-1-t', R-1-r'): the data gradient at
+// pixel x sums E at x + pad - s, so with mirrored taps it is a forward gather
+// over E with padding (T-1-pad_d, R-1-pad_h, S-1-pad_w), served by
+// GatherRowSegLoader.  The TAPS filter columns are one row of the filter (S = TAPS).
+template <typename T, int BK, int TAPS>
+struct FilterTapColsLoader {
+    const T* F;
+    int      C;          // rows
+    int      K;          // output maps
+    int      RSTK;       // elements between consecutive channels
+    FastDiv  tr_div, r_div;
+    int      TR, R;      // filter rows (t, r); R
+
+    static constexpr bool DIRECT = true;
+    static constexpr bool TILE_READS_TABLE = false;
+
+    struct Ctx { unsigned off; int kc; };
+    struct Tile { BufferRsrc rsrc; int kvalid; };
+    typedef NoWaveState Wave;
+    __device__ __forceinline__ Wave wave_init(int /*lane*/) const { return Wave{}; }
+
+    __device__ __forceinline__ Ctx prepare(int m, int kr) const
+    {
+        Ctx c;
+        const int tap = kr / BK;
+        c.kc = kr - tap * BK;
+        c.off = (m < C) ? (unsigned)(m * RSTK + (TAPS - 1 - tap) * K + c.kc) * (unsigned)sizeof(T) : NG_OOB_OFFSET;
+        return c;
+    }
+    __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/, const Wave&) const
+    {
+        const int blk = (int)tr_div.div((unsigned)kt);
+        const int tr = kt - blk * TR;
+        const int ft = (int)r_div.div((unsigned)tr);
+        const int fr = tr - ft * R;
+        const int row = (TR / R - 1 - ft) * R + (R - 1 - fr);
+        Tile t;
+        t.rsrc = make_rsrc(F + (long)row * TAPS * K + (long)blk * BK);
+        t.kvalid = K - blk * BK;
+        return t;
+    }
+    // K is a multiple of the chunk length, so a chunk is inside or outside as a whole
+    __device__ __forceinline__ unsigned offset(const Tile& t, const Ctx& c) const
+    {
+        return c.kc < t.kvalid ? c.off : NG_OOB_OFFSET;
+    }
+    __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const { return buffer_load_chunk(t.rsrc, offset(t, c)); }
+};
+
 // A operand of the blocked data gradient: the filter F[c][trs][k] in place,
 // read as rows c with the contraction (tap, k): for one tap the k values of a
 // row are contiguous, so tile (tap, block) is a contraction-contiguous tile of

@@ -146,6 +146,7 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
         int splits = std::max(conv_splits(cdiv(pl->CRST, 128) * cdiv(p.K, 128), kt, 0, 0),
                               conv_splits(cdiv(pl->CRST, 256) * cdiv(p.K, 256), kt, 0, 0));
         if (p.K <= 64 && pl->CRST <= 64) splits = std::max(splits, conv_splits(1, kt, 0, 0, 6));
+        splits = std::max(splits, conv_splits(cdiv(pl->CRST, 192) * cdiv(p.K, p.K <= 64 ? 64 : 128), kt, 0, 0));
         pl->ws_update = splits > 1 ? align_up((size_t)splits * pl->CRST * p.K * sizeof(float), 256) : 0;
     }
     *plan_out = pl;

@@ -670,6 +670,31 @@ struct SwizzledFrag<MC, Tile> {
     }
 };
 
+// A operand of a kernel whose B tile serves TAPS filter taps.  A row-contiguous
+// tile simply gets TAPS * BK lines.  A contraction-contiguous one would get lines
+// of TAPS * BK elements, which the power-of-two swizzle cannot permute, so it is
+// kept as TAPS tiles of BK elements per line, one behind the other.
+template <typename T, int LAYOUT, int ROWS, int BK, int TAPS>
+struct TapTile {
+    static constexpr bool STACKED = (LAYOUT == KC && TAPS > 1);
+    using Sub = SwizzledTile<T, LAYOUT, ROWS, STACKED ? BK : BK * TAPS>;
+    static constexpr int BYTES  = Sub::BYTES * (STACKED ? TAPS : 1);
+    static constexpr int CHUNKS = Sub::CHUNKS * (STACKED ? TAPS : 1);
+    static __device__ __forceinline__ void chunk_pos(int id, int& r, int& k)
+    {
+        if (STACKED) {
+            const int tap = id / Sub::CHUNKS;
+            Sub::chunk_pos(id - tap * Sub::CHUNKS, r, k);
+            k += tap * BK;
+        } else {
+            Sub::chunk_pos(id, r, k);
+        }
+    }
+    // byte offset of the sub-tile and the k-step inside it for k-step `step` of the whole tile
+    static constexpr int tile_of(int step, int ks) { return STACKED ? (step / ks) * Sub::BYTES : 0; }
+    static constexpr int step_of(int step, int ks) { return STACKED ? step % ks : step; }
+};
+
 // s_waitcnt immediate: at most `vm` vector-memory operations outstanding, all
 // LDS operations complete
 // 16 bytes per lane from a buffer straight into LDS: lane l of the wavefront
@@ -706,9 +731,9 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     constexpr int TAPS = LoaderTaps<BLoad>::taps;          // filter taps served by one B tile
     constexpr int TAP_COLS = LoaderTaps<BLoad>::cols;      // columns by which a tap shifts its window
     static_assert(TAPS == 1 || (LB == MC && TAP_COLS % 32 == 0), "shared taps need a row-contiguous B tile");
-    using TA = SwizzledTile<T, LA, BM, BK * TAPS>;
+    using TA = TapTile<T, LA, BM, BK, TAPS>;
     using TB = SwizzledTile<T, LB, BN + (TAPS - 1) * TAP_COLS, BK>;
-    using FA = SwizzledFrag<LA, TA>;
+    using FA = SwizzledFrag<LA, typename TA::Sub>;
     using FB = SwizzledFrag<LB, TB>;
     constexpr int CPT_A = TA::CHUNKS / NT;
     constexpr int CPT_B = TB::CHUNKS / NT;
@@ -825,7 +850,7 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     auto load_frags = [&](int stage_off, int step, Frag<T> (&a)[TM], Frag<T> (&b)[TN]) {
         const char* tile = smem + stage_off;
 #pragma unroll
-        for (int i = 0; i < TM; i++) a[i] = FA::load(tile, fa_base[i], step);
+        for (int i = 0; i < TM; i++) a[i] = FA::load(tile + TA::tile_of(step, KS), fa_base[i], TA::step_of(step, KS));
 #pragma unroll
         for (int j = 0; j < TN; j++) b[j] = FB::load(tile, fb_base[step / KS][j], step % KS);
     };

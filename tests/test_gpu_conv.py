@@ -37,6 +37,14 @@ SMALL = [
     (64, 32, 32, 4, 6, 8, 2, 3, 3, (1, 1, 1), (1, 1, 1)),          # 3-D
     (64, 64, 136, 1, 5, 8, 1, 1, 3, (0, 0, 1), (1, 1, 1)),         # one filter row
     (64, 32, 16, 1, 4, 4, 1, 3, 3, (0, 1, 3), (1, 1, 1)),          # padding wider than the filter reach
+    # the data gradient shares taps when the image rows are a multiple of four pixels and the output
+    # maps come in blocks of 32 (the taps are mirrored: two-row filter, ragged channel count)
+    (64, 72, 96, 1, 5, 12, 1, 3, 3, (0, 0, 0), (1, 1, 1)),
+    (64, 40, 32, 1, 4, 4, 1, 2, 3, (0, 1, 3), (1, 1, 1)),
+    (64, 32, 64, 3, 4, 8, 3, 2, 3, (2, 0, 1), (1, 1, 1)),          # 3-D, padding only in depth and width
+    # long pixel ranges with filter rows in multiples of 192: the weight gradient's 192-row tiles
+    (64, 64, 32, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (64, 64, 96, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
 ]
 
 
@@ -305,9 +313,10 @@ def test_deconv_layer_and_errors(ng):
 def test_bprop_with_rectifier_mask(ng, dtype):
     """bprop_conv(..., relu_mask=act) = bprop_conv followed by the reference's
     relu derivative step `grad *= act > 0` (nervanagpu/layers.py:89-91), on the
-    blocked and the row-by-row form, full and ragged tiles; strided layers refuse."""
+    blocked, the row-by-row and the shared-tap form, full and ragged tiles; strided layers refuse."""
     rng = np.random.default_rng(29)
-    for case in (SMALL[0], SMALL[2], SMALL[5], SMALL[8], SMALL[11], (16, 64, 64, 1, 20, 20, 1, 3, 3, (0, 1, 1), (1, 1, 1))):
+    for case in (SMALL[0], SMALL[2], SMALL[5], SMALL[8], SMALL[11], SMALL[21], SMALL[23],
+                 (16, 64, 64, 1, 20, 20, 1, 3, 3, (0, 1, 1), (1, 1, 1))):
         layer = _layer(ng, dtype, case)
         I, F, E = _data(layer, dtype, 31)
         act = np.maximum(rng.standard_normal(layer.dimI), 0).astype(dtype)     # about half zeros
