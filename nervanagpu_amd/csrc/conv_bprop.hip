@@ -165,6 +165,61 @@ static int bprop_shared_taps(const ConvPlan& pl, const void* F, const void* E, v
     return launch_core<T, BM, BN, BK, WM, WN, KC, MC>(al, bl, epi, p.C, ncols, TR * nblk, 1, stream, "conv bprop (shared taps)");
 }
 
+// Very few channels (a first layer): rows (channel, horizontal tap), see
+// FilterChannelTapLoader.  Strips of six output pixels from eight pixels of E.
+static bool thin_channels(const ConvPlan& pl, const void* mask)
+{
+    const ng_conv_params& p = pl.p;
+    return !mask && 3 * p.C <= 32 && p.S == 3 && p.N == 64 && p.K % 8 == 0 &&
+           p.str_d == 1 && p.str_h == 1 && p.str_w == 1;
+}
+
+// the same problem on the streaming kernel (stream_core.h): the filter, KT tiles of
+// 32 contraction rows, stays in registers; at most five channels (15 parked rows)
+template <int KT>
+static int bprop_thin_stream(const ConvPlan& pl, const void* F, const void* E, void* gradI, float alpha, hipStream_t stream)
+{
+    typedef _Float16 T;
+    constexpr int BN = 512, BK = 32, OUT_PIX = 6;
+    const ng_conv_params& p = pl.p;
+    const int strips = cdiv(p.W, OUT_PIX);
+    const int tiles = p.D * p.H * strips;
+    const int nblk = cdiv(p.K, BK);
+    FilterChannelTapLoader<T, BK> al{(const T*)F, 3 * p.C, p.K, pl.RST * p.K, FastDiv::make((unsigned)nblk), nblk};
+    HaloStripGather<T, BK, BN, OUT_PIX> bg{(const T*)E, p.M, p.P, p.Q, p.N, p.M * p.P * p.Q * p.N, tiles * BN,
+                                           FastDiv::make((unsigned)strips), FastDiv::make((unsigned)p.H), strips, p.H,
+                                           p.pad_d, p.pad_h, p.pad_w,
+                                           FastDiv::make((unsigned)nblk), FastDiv::make((unsigned)p.R), nblk, p.R, p.K};
+    ShiftSumStoreEpilogue<T, BN, OUT_PIX, 16> epi{(T*)gradI, 3 * p.C, (long)p.D * p.H * p.W * p.N, p.W, p.N,
+                                                  FastDiv::make((unsigned)strips), strips, alpha};
+    launch_stream<T, 32, BN, BK, 4, KT, KC, 3>(al, bg, epi, tiles, 1, stream);
+    NG_CHECK_LAUNCH("conv bprop (channel-tap rows, streamed)");
+    return 0;
+}
+
+static int bprop_thin(const ConvPlan& pl, const void* F, const void* E, void* gradI, float alpha, hipStream_t stream)
+{
+    typedef _Float16 T;
+    constexpr int BN = 512, BK = 32, OUT_PIX = 6;
+    const ng_conv_params& p = pl.p;
+    const int strips = cdiv(p.W, OUT_PIX);
+    const int tiles = p.D * p.H * strips;
+    const int TR = p.T * p.R, nblk = cdiv(p.K, BK);
+    if (p.C <= 5 && tiles >= device_cu_count()) {
+        if (TR * nblk == 3) return bprop_thin_stream<3>(pl, F, E, gradI, alpha, stream);
+        if (TR * nblk == 6) return bprop_thin_stream<6>(pl, F, E, gradI, alpha, stream);
+    }
+    FilterChannelTapLoader<T, BK> al{(const T*)F, 3 * p.C, p.K, pl.RST * p.K, FastDiv::make((unsigned)nblk), nblk};
+    HaloStripLoader<T, BK, BN, OUT_PIX> bl{(const T*)E, p.M, p.P, p.Q, p.N, p.M * p.P * p.Q * p.N, tiles * BN,
+                                           FastDiv::make((unsigned)strips), FastDiv::make((unsigned)p.H), strips, p.H,
+                                           p.pad_d, p.pad_h, p.pad_w,
+                                           FastDiv::make((unsigned)nblk), FastDiv::make((unsigned)p.R), nblk, p.R, p.K};
+    ShiftSumStoreEpilogue<T, BN, OUT_PIX> epi{(T*)gradI, 3 * p.C, (long)p.D * p.H * p.W * p.N, p.W, p.N,
+                                              FastDiv::make((unsigned)strips), strips, alpha};
+    return launch_core<T, 32, BN, BK, 1, 2, KC, MC>(al, bl, epi, 3 * p.C, tiles * BN, TR * nblk, 1, stream,
+                                                    "conv bprop (channel-tap rows)");
+}
+
 template <bool BLOCKED>
 static int bprop_class_h(const ConvPlan& pl, const BpropClass& c, const void* F, const _Float16* Fs, const void* E,
                          void* gradI, float alpha, const void* mask, hipStream_t st)
@@ -199,6 +254,7 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
         NG_CHECK_LAUNCH("filter relayout");
     }
     if constexpr (sizeof(T) == 2) {
+        if (thin_channels(pl, mask)) return bprop_thin(pl, F, E, gradI, alpha, stream);
         if (shares_taps(pl)) {
             switch (pick_row_tile(p.C, p.D * p.H * p.W * p.N, 256)) {
             case 256: return bprop_shared_taps<256, 2, 4>(pl, F, E, gradI, alpha, mask, stream);

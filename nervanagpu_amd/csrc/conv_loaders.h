@@ -433,6 +433,298 @@ struct FilterTapColsLoader {
     __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const { return buffer_load_chunk(t.rsrc, offset(t, c)); }
 };
 
+// Data gradient of a layer with very few channels (3 * C <= 32, filter rows of
+// three taps, unit strides, N = 64).  Rows are (c, s): G[(c,s)][z,y,x'] = sum over
+// (t, r, k) of F[c,t,r,s,k] * E[k, z+pad_d-t, y+pad_h-r, x'], so the horizontal
+// tap never enters the contraction (192 deep for 64 output maps instead of 576)
+// and the 32 rows of a matrix instruction hold three taps of every channel
+// instead of the channels alone.  The epilogue adds the three taps of a channel at
+// columns shifted by one pixel each: gradI[c,z,y,x] = sum_s G[(c,s)][z,y,x+pad_w-s].
+//
+// A workgroup's tile is one strip of an image row: HALO_PIX = OUT_PIX + 2 pixels
+// of E (x' from x0 + pad_w - 2) give OUT_PIX pixels of the gradient from x0 =
+// OUT_PIX * (strip index).  Column tiles are numbered (z*H + y) * strips + strip.
+//
+// A operand: line kc of tile (t, r, block) for row (c, s) is F[c][t][r][s][block*BK + kc].
+template <typename T, int BK>
+struct FilterChannelTapLoader {
+    const T* F;
+    int      rows;       // 3 * C
+    int      K;
+    int      RSTK;       // elements between consecutive channels
+    FastDiv  blk_div;    // tile index -> filter row (t, r); blocks of output maps are the fast index
+    int      nblk;
+
+    static constexpr bool DIRECT = true;
+    static constexpr bool TILE_READS_TABLE = false;
+
+    struct Ctx { unsigned off; int kc; };
+    struct Tile { BufferRsrc rsrc; int kvalid; };
+    typedef NoWaveState Wave;
+    __device__ __forceinline__ Wave wave_init(int /*lane*/) const { return Wave{}; }
+
+    __device__ __forceinline__ Ctx prepare(int m, int kc) const
+    {
+        Ctx c;
+        const int ch = m / 3, tap = m - ch * 3;
+        c.kc = kc;
+        c.off = (m < rows) ? (unsigned)(ch * RSTK + tap * K + kc) * (unsigned)sizeof(T) : NG_OOB_OFFSET;
+        return c;
+    }
+    __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/, const Wave&) const
+    {
+        const int tr = (int)blk_div.div((unsigned)kt);
+        const int blk = kt - tr * nblk;
+        Tile t;
+        t.rsrc = make_rsrc(F + (long)tr * 3 * K + (long)blk * BK);
+        t.kvalid = K - blk * BK;
+        return t;
+    }
+    __device__ __forceinline__ unsigned offset(const Tile& t, const Ctx& c) const
+    {
+        return c.kc < t.kvalid ? c.off : NG_OOB_OFFSET;
+    }
+    __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const { return buffer_load_chunk(t.rsrc, offset(t, c)); }
+};
+
+// B operand of the same kernel: column r of tile (z, y, strip) is pixel
+// x' = strip*OUT_PIX + pad_w - 2 + r / N of E row (z + pad_d - t, y + pad_h - r_f),
+// image r % N; everything outside E reads zero.
+template <typename T, int BK, int BN, int OUT_PIX>
+struct HaloStripLoader {
+    const T* E;
+    int      M, P, Q;        // extents of E
+    int      N;
+    int      row_stride;     // elements between consecutive output maps (M*P*Q*N)
+    int      ncols;          // tiles * BN
+    FastDiv  strip_div, h_div;
+    int      strips, H;      // strips per image row; image rows per depth slice
+    int      pad_d, pad_h, pad_w;
+    FastDiv  blk_div, r_div;
+    int      nblk, R, K;
+
+    static constexpr bool DIRECT = true;
+    static constexpr bool TILE_READS_TABLE = false;
+
+    struct Ctx { int base, z0, y0, kr; };
+    struct Tile { BufferRsrc rsrc; int toff, dz, dy, k0; };
+    typedef NoWaveState Wave;
+    __device__ __forceinline__ Wave wave_init(int /*lane*/) const { return Wave{}; }
+
+    __device__ __forceinline__ Ctx prepare(int col, int kr) const
+    {
+        Ctx c;
+        c.kr = kr;
+        c.base = 0; c.z0 = c.y0 = NG_FAR;
+        if (col >= ncols) return c;
+        const int tile = col / BN, r = col - tile * BN;
+        const int zy = (int)strip_div.div((unsigned)tile);
+        const int strip = tile - zy * strips;
+        const int z = (int)h_div.div((unsigned)zy);
+        const int y = zy - z * H;
+        const int pix = r / N, nn = r - pix * N;
+        const int x = strip * OUT_PIX + pad_w - 2 + pix;
+        if ((unsigned)x >= (unsigned)Q) return c;
+        c.z0 = z + pad_d; c.y0 = y + pad_h;
+        c.base = ((c.z0 * P + c.y0) * Q + x) * N + nn + kr * row_stride;
+        return c;
+    }
+    __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/, const Wave&) const
+    {
+        Tile t;
+        t.rsrc = make_rsrc(E);
+        const int tr = (int)blk_div.div((unsigned)kt);
+        const int blk = kt - tr * nblk;
+        const int ft = (int)r_div.div((unsigned)tr);
+        const int fr = tr - ft * R;
+        t.dz = -ft; t.dy = -fr;
+        t.toff = (t.dz * P + t.dy) * Q * N + blk * BK * row_stride;
+        t.k0 = K - blk * BK;
+        return t;
+    }
+    __device__ __forceinline__ unsigned offset(const Tile& t, const Ctx& c) const
+    {
+        const bool ok = ((unsigned)(c.z0 + t.dz) < (unsigned)M) & ((unsigned)(c.y0 + t.dy) < (unsigned)P) & (c.kr < t.k0);
+        const unsigned off = (unsigned)(c.base + t.toff) * (unsigned)sizeof(T);
+        return ok ? off : NG_OOB_OFFSET;
+    }
+    __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const { return buffer_load_chunk(t.rsrc, offset(t, c)); }
+};
+
+// Epilogue of the same kernel: g holds the fp32 tile, rows (c, s), BN columns
+// (HALO_PIX pixels x N images).  Output pixel i of the strip adds column block
+// i + 2 - s of row (c, s) over the three taps, in that order; one rounding.
+template <typename T, int BN, int OUT_PIX, int MAX_ROWS_ = 32>
+struct ShiftSumStoreEpilogue {
+    static constexpr bool WHOLE_TILE = true;
+    static constexpr int MAX_ROWS = MAX_ROWS_;   // rows the streaming kernel parks (3 * C at most)
+    typedef typename StoreBits<T>::bits_t bits_t;
+    T*      out;
+    int     rows;          // 3 * C
+    long    chan_stride;   // D*H*W*N
+    int     W, N;
+    FastDiv strip_div;
+    int     strips;
+    float   alpha;
+
+    __device__ __forceinline__ const void* base() const { return out; }
+    // the same for the streaming kernel: exactly one descriptor store per thread
+    // (3 * C <= MAX_ROWS <= 16 keeps the 8-element pieces of a strip within 256
+    // threads); threads without a piece store out of range
+    static constexpr int STORES_PER_THREAD = 1;
+    __device__ __forceinline__ void tile_buffer(BufferRsrc rsrc, const float* g, int tid, int n0) const
+    {
+        const int t = n0 / BN;
+        const int zy = (int)strip_div.div((unsigned)t);
+        const int x0 = (t - zy * strips) * OUT_PIX;
+        const int per_chan = OUT_PIX * (N / 8);
+        const int chans = rows / 3;
+        const int c = tid / per_chan, rem = tid - c * per_chan;
+        const int i = rem / (N / 8), n8 = (rem - i * (N / 8)) * 8;
+        const int x = x0 + i;
+        const int cr = min(c, chans - 1);   // keeps the LDS reads of idle threads inside the parked rows
+        float sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int s = 0; s < 3; s++) {
+            const float* p = g + (cr * 3 + s) * BN + (i + 2 - s) * N + n8;
+            const float4_t lo = *reinterpret_cast<const float4_t*>(p);
+            const float4_t hi = *reinterpret_cast<const float4_t*>(p + 4);
+#pragma unroll
+            for (int q = 0; q < 4; q++) { sum[q] += lo[q]; sum[4 + q] += hi[q]; }
+        }
+        bits_t r[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) r[q] = StoreBits<T>::round(sum[q] * alpha, 0, 0, 0, 0);
+        const long e = (long)c * chan_stride + ((long)zy * W + x) * N + n8;
+        const unsigned off = (c < chans && x < W) ? (unsigned)e * 2u : NG_OOB_OFFSET;
+        buffer_store_chunk(rsrc, off, *reinterpret_cast<const uint4_t*>(r));
+    }
+
+    __device__ __forceinline__ void tile(const float* g, int tid, int nthreads, int n0) const
+    {
+        const int t = n0 / BN;
+        const int zy = (int)strip_div.div((unsigned)t);
+        const int x0 = (t - zy * strips) * OUT_PIX;
+        const int per_chan = OUT_PIX * (N / 8);
+        const int total = (rows / 3) * per_chan;
+        for (int e = tid; e < total; e += nthreads) {
+            const int c = e / per_chan, rem = e - c * per_chan;
+            const int i = rem / (N / 8), n8 = (rem - i * (N / 8)) * 8;
+            const int x = x0 + i;
+            if (x >= W) continue;
+            float sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int s = 0; s < 3; s++) {
+                const float* p = g + (c * 3 + s) * BN + (i + 2 - s) * N + n8;
+                const float4_t lo = *reinterpret_cast<const float4_t*>(p);
+                const float4_t hi = *reinterpret_cast<const float4_t*>(p + 4);
+#pragma unroll
+                for (int q = 0; q < 4; q++) { sum[q] += lo[q]; sum[4 + q] += hi[q]; }
+            }
+            bits_t r[8];
+#pragma unroll
+            for (int q = 0; q < 8; q++) r[q] = StoreBits<T>::round(sum[q] * alpha, 0, 0, 0, 0);
+            bits_t* dst = reinterpret_cast<bits_t*>(out) + (long)c * chan_stride + ((long)zy * W + x) * N + n8;
+            *reinterpret_cast<uint4_t*>(dst) = *reinterpret_cast<const uint4_t*>(r);
+        }
+    }
+};
+
+// ---- gather functors of the streaming kernel (stream_core.h) --------------------
+// Both describe a chunk as base(column) + off(contraction row), valid when the
+// column's pixel shifted by the row's (dz, dy, dx) lies inside the tensor.
+struct StreamFixed { int off, dz, dy, dx; };
+struct StreamCol { int base, z0, y0, x0; };
+
+template <typename T>
+__device__ __forceinline__ unsigned stream_offset(const StreamFixed& f, const StreamCol& c, int lim_d, int lim_h, int lim_w)
+{
+    const bool ok = ((unsigned)(c.z0 + f.dz) < (unsigned)lim_d) & ((unsigned)(c.y0 + f.dy) < (unsigned)lim_h) &
+                    ((unsigned)(c.x0 + f.dx) < (unsigned)lim_w);
+    const unsigned off = (unsigned)(c.base + f.off) * (unsigned)sizeof(T);
+    return ok ? off : NG_OOB_OFFSET;
+}
+
+// forward convolution, contraction rows (c, t, r, s) from the flat tap table
+template <typename T>
+struct FlatTapGather {
+    const T*        X;
+    const TapEntry* tab;
+    int             J;
+    PixelLattice    lat;
+    int             gs_d, gs_h, gs_w;
+    int             lim_d, lim_h, lim_w;
+    typedef StreamFixed Fixed;
+    typedef StreamCol Col;
+
+    __device__ __forceinline__ Fixed fixed(int j) const
+    {
+        if (j >= J) return Fixed{0, NG_FAR, NG_FAR, NG_FAR};
+        const TapEntry e = tab[j];
+        return Fixed{e.off, e.dz, e.dy, e.dx};
+    }
+    __device__ __forceinline__ Col col(int c) const
+    {
+        if (c >= lat.ncols) return Col{0, NG_FAR, NG_FAR, NG_FAR};
+        int iz, iy, ix, nn;
+        lat.split(c, iz, iy, ix, nn);
+        Col o;
+        o.z0 = iz * gs_d; o.y0 = iy * gs_h; o.x0 = ix * gs_w;
+        o.base = ((o.z0 * lim_h + o.y0) * lim_w + o.x0) * lat.N + nn;
+        return o;
+    }
+    __device__ __forceinline__ unsigned offset(const Fixed& f, const Col& c) const
+    {
+        return stream_offset<T>(f, c, lim_d, lim_h, lim_w);
+    }
+};
+
+// data gradient with rows (channel, horizontal tap): contraction rows
+// ((t, r), output map), columns the halo strips of HaloStripLoader
+template <typename T, int BK, int BN, int OUT_PIX>
+struct HaloStripGather {
+    const T* X;              // E
+    int      M, P, Q, N;
+    int      row_stride;     // M*P*Q*N
+    int      ncols;
+    FastDiv  strip_div, h_div;
+    int      strips, H;
+    int      pad_d, pad_h, pad_w;
+    FastDiv  blk_div, r_div;
+    int      nblk, R, K;
+    typedef StreamFixed Fixed;
+    typedef StreamCol Col;
+
+    __device__ __forceinline__ Fixed fixed(int j) const
+    {
+        const int kt = j / BK, kr = j - kt * BK;
+        const int tr = (int)blk_div.div((unsigned)kt);
+        const int kk = (kt - tr * nblk) * BK + kr;
+        const int ft = (int)r_div.div((unsigned)tr);
+        const int fr = tr - ft * R;
+        if (kk >= K) return Fixed{0, NG_FAR, NG_FAR, NG_FAR};
+        return Fixed{(-ft * P - fr) * Q * N + kk * row_stride, -ft, -fr, 0};
+    }
+    __device__ __forceinline__ Col col(int c) const
+    {
+        if (c >= ncols) return Col{0, NG_FAR, NG_FAR, NG_FAR};
+        const int tile = c / BN, r = c - tile * BN;
+        const int zy = (int)strip_div.div((unsigned)tile);
+        const int strip = tile - zy * strips;
+        const int z = (int)h_div.div((unsigned)zy);
+        const int y = zy - z * H;
+        const int pix = r / N, nn = r - pix * N;
+        Col o;
+        o.z0 = z + pad_d; o.y0 = y + pad_h; o.x0 = strip * OUT_PIX + pad_w - 2 + pix;
+        o.base = ((o.z0 * P + o.y0) * Q + o.x0) * N + nn;
+        return o;
+    }
+    __device__ __forceinline__ unsigned offset(const Fixed& f, const Col& c) const
+    {
+        return stream_offset<T>(f, c, M, P, Q);
+    }
+};
+
 // A operand of the blocked data gradient: the filter F[c][trs][k] in place,
 // read as rows c with the contraction (tap, k): for one tap the k values of a
 // row are contiguous, so tile (tap, block) is a contraction-contiguous tile of

@@ -3,6 +3,7 @@
 #pragma once
 
 #include "conv_loaders.h"
+#include "stream_core.h"
 
 #include <algorithm>
 #include <vector>

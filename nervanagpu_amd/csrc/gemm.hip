@@ -119,6 +119,9 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
         // short contractions are all prologue and epilogue: half-depth tiles halve
         // the LDS footprint, so more workgroups overlap their loads and stores
         if (k_tiles <= 4) return launch_layout<_Float16, 128, 128, 32, 2, 2, true>(g, sr_bits);
+        // about one workgroup per CU: no second workgroup overlaps the wait for a
+        // tile, a third stage does (2048^3: 29.5 -> 25.4 us)
+        if (4 * tiles128 <= 5 * cus && k_tiles >= 16) return launch_layout<_Float16, 128, 128, 64, 2, 2, true, 3>(g, sr_bits);
         return launch_layout<_Float16, 128, 128, 64, 2, 2, true>(g, sr_bits);
     }
     if (g.n <= 128) return launch_layout<_Float16, 64, 128, 64, 2, 2, true>(g, sr_bits);

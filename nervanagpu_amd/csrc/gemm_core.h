@@ -174,6 +174,14 @@ __device__ __forceinline__ uint4_t buffer_load_chunk(BufferRsrc rsrc, unsigned b
     return __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)byte_offset, 0, 0);
 }
 
+// 16-byte store through a descriptor: an offset at or beyond its range is dropped
+// by the hardware, so a lane with nothing to store still takes part and every
+// wavefront issues the same number of store instructions
+__device__ __forceinline__ void buffer_store_chunk(BufferRsrc rsrc, unsigned byte_offset, uint4_t v)
+{
+    __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, (int)byte_offset, 0, 0);
+}
+
 // Loader protocol used by the core (all three calls are inlined):
 //   Ctx  prepare(r, kc)      once per 16-byte chunk a thread owns: r = absolute
 //                            row of the operand, kc = contraction offset of the
@@ -203,6 +211,13 @@ struct NoWaveState {};
 // kernel is TAPS * BK deep (tap-major).
 template <class L, class = void> struct LoaderTaps { static constexpr int taps = 1, cols = 0; };
 template <class L> struct LoaderTaps<L, std::enable_if_t<(L::TAPS > 1)>> { static constexpr int taps = L::TAPS, cols = L::TAP_COLS; };
+
+// An epilogue that combines values across the columns of a workgroup's tile
+// declares `static constexpr bool WHOLE_TILE = true` and tile(g, tid, nthreads,
+// n0): the kernel (one row block of 32 rows) parks the fp32 tile in LDS, row-major
+// with BN columns, before calling it.
+template <class E, class = void> struct EpilogueWholeTile { static constexpr bool value = false; };
+template <class E> struct EpilogueWholeTile<E, std::enable_if_t<E::WHOLE_TILE>> { static constexpr bool value = true; };
 
 // loaders that can step a tile descriptor to the next contraction tile declare
 // `static constexpr bool INCREMENTAL = true` and advance(Tile&, bk)
@@ -921,11 +936,16 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
             const Frag<T> (&ca)[TM] = fa[(NSTEP - 1) & 1];
             const Frag<T> (&cb)[TN] = fb[(NSTEP - 1) & 1];
             constexpr int PER = (N_CHUNKS + N_MFMA - 1) / N_MFMA;
+            constexpr int FPM = (TM + TN + N_MFMA - 1) / N_MFMA;   // fragment reads per MFMA
 #pragma unroll
             for (int m = 0; m < N_MFMA; m++) {
                 mfma_step(ca[m / TN], cb[m % TN], acc[m / TN][m % TN]);
-                if (m < TM) na[m < TM ? m : 0] = FA::load(tile, fa_base[m < TM ? m : 0], 0);
-                else if (m < TM + TN) nb[m - TM < TN ? (m >= TM ? m - TM : 0) : 0] = FB::load(tile, fb_base[0][m - TM < TN ? (m >= TM ? m - TM : 0) : 0], 0);
+#pragma unroll
+                for (int q = 0; q < FPM; q++) {
+                    const int f = m * FPM + q;   // fragment of tile t+1 read behind this MFMA
+                    if (f < TM) na[f < TM ? f : 0] = FA::load(tile, fa_base[f < TM ? f : 0], 0);
+                    else if (f < TM + TN) nb[f >= TM && f < TM + TN ? f - TM : 0] = FB::load(tile, fb_base[0][f >= TM && f < TM + TN ? f - TM : 0], 0);
+                }
 #pragma unroll
                 for (int q = 0; q < PER; q++) {
                     const int c = m * PER + q;
@@ -962,9 +982,25 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
         multiply(fa[(NSTEP - 1) & 1], fb[(NSTEP - 1) & 1]);
     }
 
-    char* stage = smem + wave * EPI_BYTES;
     __syncthreads();
-    EpilogueBands<TM, TN, WTN, EPITCH, 0>::run(acc, stage, lane, m0 + wm * (BM / WM), n0 + wn * WTN, z, split, epi);
+    if constexpr (EpilogueWholeTile<Epi>::value) {
+        static_assert(BM == 32 && WM == 1, "whole-tile epilogues take one block of 32 rows");
+        static_assert(32 * BN * 4 <= SMEM_BYTES, "the fp32 tile must fit the LDS of the stages");
+        float* g = reinterpret_cast<float*>(smem);
+        const int nrows = epi.rows;
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+                if (row < nrows) g[row * BN + wn * WTN + j * 32 + (lane & 31)] = acc[0][j][v];
+            }
+        __syncthreads();
+        epi.tile(g, tid, NT, n0);
+    } else {
+        char* stage = smem + wave * EPI_BYTES;
+        EpilogueBands<TM, TN, WTN, EPITCH, 0>::run(acc, stage, lane, m0 + wm * (BM / WM), n0 + wn * WTN, z, split, epi);
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -1032,6 +1068,7 @@ struct ScaleStoreEpilogue {
     // the layer whose activations the mask holds)
     const T* mask = nullptr;
 
+    __device__ __forceinline__ const void* base() const { return C; }
     __device__ __forceinline__ bool masked_out(long offset) const
     {
         return !(StoreBits<T>::widen(reinterpret_cast<const bits_t*>(mask)[offset]) > 0.0f);
@@ -1065,6 +1102,23 @@ struct ScaleStoreEpilogue {
         if (beta != 0.0f) v += beta * StoreBits<T>::widen(*p);
         const bits_t r = StoreBits<T>::round(v, sr_bits, seed, stream, rng_index(i, j, z));
         *p = (mask && masked_out(offset)) ? (bits_t)0 : r;
+    }
+    // The plain case of store8 (16-bit elements, rows of C 16-byte aligned, no beta,
+    // nearest rounding, no mask, one matrix) as a descriptor store on C: positions
+    // outside the matrix are dropped by the hardware instead of branched around.
+    __device__ __forceinline__ void store8_buffer(BufferRsrc rsrc, int i, int j0, const float (&acc)[8]) const
+    {
+        static_assert(sizeof(bits_t) == 2, "descriptor stores are written for 16-bit outputs");
+        bits_t out[8];
+        if (relu) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) out[e] = StoreBits<T>::round(fmaxf(acc[e] * alpha, 0.0f), 0, 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) out[e] = StoreBits<T>::round(acc[e] * alpha, 0, 0, 0, 0);
+        }
+        const unsigned off = (i < m && j0 < n) ? ((unsigned)i * (unsigned)ldc + (unsigned)j0) * 2u : NG_OOB_OFFSET;
+        buffer_store_chunk(rsrc, off, *reinterpret_cast<const uint4_t*>(out));
     }
     __device__ __forceinline__ void store8(int i, int j0, int z, int /*split*/, const float (&acc)[8]) const
     {

