@@ -36,22 +36,33 @@ static int fprop_tile(const ConvPlan& pl, const void* I, const void* F, void* O,
 static bool shares_taps(const ConvPlan& pl)
 {
     const ng_conv_params& p = pl.p;
-    return p.S == 3 && p.N == 64 && p.Q % 4 == 0 && p.C % 32 == 0 &&
+    // image rows that are not a whole number of tiles are padded to one if that
+    // wastes at most a twelfth of the columns (the epilogue folds them away)
+    const int qpad = cdiv(p.Q, 4) * 4;
+    return p.S == 3 && (p.N == 64 || p.N == 32) && 12 * (qpad - p.Q) <= qpad && p.C % 32 == 0 &&
            p.str_d == 1 && p.str_h == 1 && p.str_w == 1;
 }
 
-template <int BM, int WM, int WN>
+// COLS = N images per pixel; a tile of BN = 4 * COLS columns is four output pixels
+template <int BM, int WM, int WN, int BN = 256, int COLS = 64>
 static int fprop_shared_taps(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags,
                              hipStream_t stream)
 {
     typedef _Float16 T;
-    constexpr int BN = 256, BK = 32, TAPS = 3, COLS = 64;
+    constexpr int BK = 32, TAPS = 3;
+    static_assert(BN == 4 * COLS, "four output pixels per tile");
     const ng_conv_params& p = pl.p;
-    const int ncols = p.M * p.P * p.Q * p.N;
+    const int qpad = cdiv(p.Q, 4) * 4;
+    const int ncols = p.M * p.P * qpad * p.N;           // the kernel's columns: padded image rows
+    const int out_cols = p.M * p.P * p.Q * p.N;
     const int TR = p.T * p.R, nblk = cdiv(p.C, BK);
-    ScaleStoreEpilogue<T> epi{(T*)O, 0, ncols, p.K, ncols, alpha, 0.0f, (flags & NG_FLAG_RELU) ? 1u : 0u, 0u, 0u, 0u, 1u};
+    ScaleStoreEpilogue<T> epi{(T*)O, 0, out_cols, p.K, out_cols, alpha, 0.0f, (flags & NG_FLAG_RELU) ? 1u : 0u, 0u, 0u, 0u, 1u};
+    if (qpad != p.Q) {
+        epi.fold_from = qpad * p.N; epi.fold_to = p.Q * p.N;
+        epi.fold_div = FastDiv::make((unsigned)epi.fold_from);
+    }
     FilterTapRowLoader<T, BK, TAPS> al{(const T*)F, p.K, pl.RST * p.K, FastDiv::make((unsigned)TR), TR, p.C};
-    GatherRowSegLoader<T, BK, TAPS, COLS> bl{(const T*)I, PixelLattice::make(p.N, ncols, p.Q, p.P * p.Q), p.D, p.H, p.W,
+    GatherRowSegLoader<T, BK, TAPS, COLS> bl{(const T*)I, PixelLattice::make(p.N, ncols, qpad, p.P * qpad), p.D, p.H, p.W,
                                              p.pad_d, p.pad_h, p.pad_w, p.D * p.H * p.W * p.N,
                                              FastDiv::make((unsigned)TR), FastDiv::make((unsigned)p.R), TR, p.R, p.C};
     return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, epi, p.K, ncols, TR * nblk, 1, stream, "conv fprop (shared taps)");
@@ -90,8 +101,11 @@ template <typename TIN, bool BLOCKED>
 static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags, hipStream_t st)
 {
     if constexpr (BLOCKED && std::is_same<TIN, _Float16>::value) {
-        if (shares_taps(pl)) {
-            switch (pick_row_tile(pl.p.K, pl.p.M * pl.p.P * pl.p.Q * pl.p.N, 256)) {
+        if (shares_taps(pl) && pl.p.N == 32) {
+            // 32 images: 128-column tiles; 128 rows on four wavefronts
+            if (pl.p.K >= 128) return fprop_shared_taps<128, 2, 2, 128, 32>(pl, I, F, O, alpha, flags, st);
+        } else if (shares_taps(pl)) {
+            switch (pick_row_tile(pl.p.K, pl.p.M * pl.p.P * cdiv(pl.p.Q, 4) * 4 * pl.p.N, 256)) {
             case 256: return fprop_shared_taps<256, 2, 4>(pl, I, F, O, alpha, flags, st);
             case 128: return fprop_shared_taps<128, 2, 4>(pl, I, F, O, alpha, flags, st);
             default:  return fprop_shared_taps<64, 1, 4>(pl, I, F, O, alpha, flags, st);

@@ -620,10 +620,13 @@ struct SwizzledTile {
     static constexpr int BYTES  = PITCH * LINES;
     static constexpr int CHUNKS = ROWS * BK / EPC;
     static constexpr int LP     = (CPR >= 16) ? 1 : 16 / CPR;               // lines per 256 bytes
-    static constexpr int GROUPS = (CPR / 4 < 4) ? CPR / 4 : 4;              // MC: 64-byte groups permuted
+    // MC: 64-byte groups permuted among themselves; the permuted span (GROUPS * 64
+    // bytes) must divide the line, so lines of 24 chunks permute pairs of groups
+    static constexpr int GROUPS = (CPR % 16 == 0) ? 4 : (CPR % 8 == 0) ? 2 : 1;
     static_assert(sizeof(T) == 2, "direct LDS tiles are implemented for 16-bit elements");
     static_assert(LAYOUT == MC || CPR <= 16, "contraction-contiguous lines longer than 256 bytes are not swizzled");
     static_assert(LAYOUT == KC || CPR >= 8, "row-contiguous tiles need at least 64 rows");
+    static_assert(LAYOUT == KC || CPR % (GROUPS * 4) == 0, "the group permutation must stay inside a line");
 
     // KC: 16 consecutive rows read the same logical chunk -> spread them over the
     //     16 chunk slots of a 256-byte bank period.
@@ -1067,6 +1070,12 @@ struct ScaleStoreEpilogue {
     // element is not positive are stored as zero (the rectifier derivative of
     // the layer whose activations the mask holds)
     const T* mask = nullptr;
+    // Optional column fold.  The kernel's columns are rows of fold_from columns of
+    // which only the first fold_to exist in C (image rows padded to a whole number
+    // of tiles): column q*fold_from + r goes to q*fold_to + r, r >= fold_to to nowhere.
+    // n stays the column count of C.  Groups of 8 columns never straddle a fold.
+    int      fold_from = 0, fold_to = 0;
+    FastDiv  fold_div = FastDiv{0, 0};
 
     __device__ __forceinline__ const void* base() const { return C; }
     __device__ __forceinline__ bool masked_out(long offset) const
@@ -1122,6 +1131,11 @@ struct ScaleStoreEpilogue {
     }
     __device__ __forceinline__ void store8(int i, int j0, int z, int /*split*/, const float (&acc)[8]) const
     {
+        if (fold_from) {
+            const int q = (int)fold_div.div((unsigned)j0), r = j0 - q * fold_from;
+            if (r >= fold_to) return;
+            j0 = q * fold_to + r;
+        }
         if (i >= m || j0 >= n) return;
         constexpr int NV = (int)sizeof(bits_t) * 8 / 16;   // 16-byte pieces per 8 elements
         const long offset = (long)z * ldcz + (long)i * ldc + j0;
