@@ -491,6 +491,7 @@ def profile_cases(ng):
     for which in ("fprop", "bprop", "update"):
         out["conv64_" + which] = lambda which=which: conv(64, 224, 64, which)
         out["conv512_" + which] = lambda which=which: conv(512, 28, 512, which)
+        out["conv3_" + which] = lambda which=which: conv(3, 224, 64, which)
 
     def pool(which):
         layer = ng.pool_layer(np.float16, "max", 128, 256, 1, 56, 56, 1, 1, 3, 3, 0, 0, 0, 0, 1, 1, 2, 2)

@@ -187,12 +187,12 @@ static int bprop_thin_stream(const ConvPlan& pl, const void* F, const void* E, v
     const int nblk = cdiv(p.K, BK);
     FilterChannelTapLoader<T, BK> al{(const T*)F, 3 * p.C, p.K, pl.RST * p.K, FastDiv::make((unsigned)nblk), nblk};
     HaloStripGather<T, BK, BN, OUT_PIX> bg{(const T*)E, p.M, p.P, p.Q, p.N, p.M * p.P * p.Q * p.N, tiles * BN,
-                                           FastDiv::make((unsigned)strips), FastDiv::make((unsigned)p.H), strips, p.H,
+                                           FastDiv::make((unsigned)(p.D * p.H)), FastDiv::make((unsigned)p.H), p.D * p.H, p.H,
                                            p.pad_d, p.pad_h, p.pad_w,
                                            FastDiv::make((unsigned)nblk), FastDiv::make((unsigned)p.R), nblk, p.R, p.K};
     ShiftSumStoreEpilogue<T, BN, OUT_PIX, 16> epi{(T*)gradI, 3 * p.C, (long)p.D * p.H * p.W * p.N, p.W, p.N,
-                                                  FastDiv::make((unsigned)strips), strips, alpha};
-    launch_stream<T, 32, BN, BK, 4, KT, KC, 3>(al, bg, epi, tiles, 1, stream);
+                                                  FastDiv::make((unsigned)(p.D * p.H)), p.D * p.H, alpha};
+    launch_stream<T, 32, BN, BK, 4, KT, KC, 2>(al, bg, epi, tiles, 2, stream);
     NG_CHECK_LAUNCH("conv bprop (channel-tap rows, streamed)");
     return 0;
 }
@@ -211,11 +211,11 @@ static int bprop_thin(const ConvPlan& pl, const void* F, const void* E, void* gr
     }
     FilterChannelTapLoader<T, BK> al{(const T*)F, 3 * p.C, p.K, pl.RST * p.K, FastDiv::make((unsigned)nblk), nblk};
     HaloStripLoader<T, BK, BN, OUT_PIX> bl{(const T*)E, p.M, p.P, p.Q, p.N, p.M * p.P * p.Q * p.N, tiles * BN,
-                                           FastDiv::make((unsigned)strips), FastDiv::make((unsigned)p.H), strips, p.H,
+                                           FastDiv::make((unsigned)(p.D * p.H)), FastDiv::make((unsigned)p.H), p.D * p.H, p.H,
                                            p.pad_d, p.pad_h, p.pad_w,
                                            FastDiv::make((unsigned)nblk), FastDiv::make((unsigned)p.R), nblk, p.R, p.K};
     ShiftSumStoreEpilogue<T, BN, OUT_PIX> epi{(T*)gradI, 3 * p.C, (long)p.D * p.H * p.W * p.N, p.W, p.N,
-                                              FastDiv::make((unsigned)strips), strips, alpha};
+                                              FastDiv::make((unsigned)(p.D * p.H)), p.D * p.H, alpha};
     return launch_core<T, 32, BN, BK, 1, 2, KC, MC>(al, bl, epi, 3 * p.C, tiles * BN, TR * nblk, 1, stream,
                                                     "conv bprop (channel-tap rows)");
 }

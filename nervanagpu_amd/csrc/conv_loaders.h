@@ -445,7 +445,19 @@ struct FilterTapColsLoader {
 // of E (x' from x0 + pad_w - 2) give OUT_PIX pixels of the gradient from x0 =
 // OUT_PIX * (strip index).  Column tiles are numbered (z*H + y) * strips + strip.
 //
+// The tiles are numbered down the image: tile = strip * (D*H) + (z*H + y), so that
+// consecutive tiles of a workgroup's run are vertically adjacent and share two of
+// the three rows of E they read (numbered along the rows, every load missed the
+// L2: FETCH_SIZE showed 3.9 x |E| for a 3x3 filter).
+//
 // A operand: line kc of tile (t, r, block) for row (c, s) is F[c][t][r][s][block*BK + kc].
+// tile -> (image row zy, strip): `rows_div` divides by the number of image rows D*H
+__device__ __forceinline__ void strip_of_tile(int tile, const FastDiv& rows_div, int img_rows, int& zy, int& strip)
+{
+    strip = (int)rows_div.div((unsigned)tile);
+    zy = tile - strip * img_rows;
+}
+
 template <typename T, int BK>
 struct FilterChannelTapLoader {
     const T* F;
@@ -497,8 +509,8 @@ struct HaloStripLoader {
     int      N;
     int      row_stride;     // elements between consecutive output maps (M*P*Q*N)
     int      ncols;          // tiles * BN
-    FastDiv  strip_div, h_div;
-    int      strips, H;      // strips per image row; image rows per depth slice
+    FastDiv  imgrow_div, h_div;
+    int      img_rows, H;    // image rows D*H; image rows per depth slice
     int      pad_d, pad_h, pad_w;
     FastDiv  blk_div, r_div;
     int      nblk, R, K;
@@ -518,8 +530,8 @@ struct HaloStripLoader {
         c.base = 0; c.z0 = c.y0 = NG_FAR;
         if (col >= ncols) return c;
         const int tile = col / BN, r = col - tile * BN;
-        const int zy = (int)strip_div.div((unsigned)tile);
-        const int strip = tile - zy * strips;
+        int zy, strip;
+        strip_of_tile(tile, imgrow_div, img_rows, zy, strip);
         const int z = (int)h_div.div((unsigned)zy);
         const int y = zy - z * H;
         const int pix = r / N, nn = r - pix * N;
@@ -563,8 +575,8 @@ struct ShiftSumStoreEpilogue {
     int     rows;          // 3 * C
     long    chan_stride;   // D*H*W*N
     int     W, N;
-    FastDiv strip_div;
-    int     strips;
+    FastDiv imgrow_div;
+    int     img_rows;      // image rows D*H
     float   alpha;
 
     __device__ __forceinline__ const void* base() const { return out; }
@@ -574,9 +586,9 @@ struct ShiftSumStoreEpilogue {
     static constexpr int STORES_PER_THREAD = 1;
     __device__ __forceinline__ void tile_buffer(BufferRsrc rsrc, const float* g, int tid, int n0) const
     {
-        const int t = n0 / BN;
-        const int zy = (int)strip_div.div((unsigned)t);
-        const int x0 = (t - zy * strips) * OUT_PIX;
+        int zy, strip;
+        strip_of_tile(n0 / BN, imgrow_div, img_rows, zy, strip);
+        const int x0 = strip * OUT_PIX;
         const int per_chan = OUT_PIX * (N / 8);
         const int chans = rows / 3;
         const int c = tid / per_chan, rem = tid - c * per_chan;
@@ -602,9 +614,9 @@ struct ShiftSumStoreEpilogue {
 
     __device__ __forceinline__ void tile(const float* g, int tid, int nthreads, int n0) const
     {
-        const int t = n0 / BN;
-        const int zy = (int)strip_div.div((unsigned)t);
-        const int x0 = (t - zy * strips) * OUT_PIX;
+        int zy, strip;
+        strip_of_tile(n0 / BN, imgrow_div, img_rows, zy, strip);
+        const int x0 = strip * OUT_PIX;
         const int per_chan = OUT_PIX * (N / 8);
         const int total = (rows / 3) * per_chan;
         for (int e = tid; e < total; e += nthreads) {
@@ -680,48 +692,64 @@ struct FlatTapGather {
 };
 
 // data gradient with rows (channel, horizontal tap): contraction rows
-// ((t, r), output map), columns the halo strips of HaloStripLoader
+// ((t, r), output map), columns the halo strips of HaloStripLoader.
+// A line of the tile (BN = 512 columns) is exactly one wavefront request, so what
+// a contraction row contributes is uniform over the wavefront, and so is the image
+// row of a column tile: those parts are kept in scalar registers and the row test
+// runs on the scalar unit; per lane remain one add and one select per request.
 template <typename T, int BK, int BN, int OUT_PIX>
 struct HaloStripGather {
+    static_assert(BN * sizeof(T) == 64 * 16, "one line of the tile per wavefront request");
     const T* X;              // E
     int      M, P, Q, N;
     int      row_stride;     // M*P*Q*N
     int      ncols;
-    FastDiv  strip_div, h_div;
-    int      strips, H;
+    FastDiv  imgrow_div, h_div;
+    int      img_rows, H;
     int      pad_d, pad_h, pad_w;
     FastDiv  blk_div, r_div;
     int      nblk, R, K;
-    typedef StreamFixed Fixed;
-    typedef StreamCol Col;
+    static constexpr bool FIXED_PER_TILE = true;
+    struct Fixed { int off, dz, dy, kleft; };            // uniform: byte offset of the tile's first row, row shifts, rows that exist
+    struct Col { unsigned base; int z0, y0; bool xok; }; // z0, y0 uniform; base, xok per lane
 
+    // j: first contraction row of a tile
     __device__ __forceinline__ Fixed fixed(int j) const
     {
-        const int kt = j / BK, kr = j - kt * BK;
+        const int kt = j / BK;
         const int tr = (int)blk_div.div((unsigned)kt);
-        const int kk = (kt - tr * nblk) * BK + kr;
+        const int k0 = (kt - tr * nblk) * BK;
         const int ft = (int)r_div.div((unsigned)tr);
         const int fr = tr - ft * R;
-        if (kk >= K) return Fixed{0, NG_FAR, NG_FAR, NG_FAR};
-        return Fixed{(-ft * P - fr) * Q * N + kk * row_stride, -ft, -fr, 0};
+        Fixed f;
+        f.off = __builtin_amdgcn_readfirstlane(((-ft * P - fr) * Q * N + k0 * row_stride) * (int)sizeof(T));
+        f.dz = __builtin_amdgcn_readfirstlane(-ft);
+        f.dy = __builtin_amdgcn_readfirstlane(-fr);
+        f.kleft = __builtin_amdgcn_readfirstlane(K - k0);
+        return f;
     }
     __device__ __forceinline__ Col col(int c) const
     {
-        if (c >= ncols) return Col{0, NG_FAR, NG_FAR, NG_FAR};
-        const int tile = c / BN, r = c - tile * BN;
-        const int zy = (int)strip_div.div((unsigned)tile);
-        const int strip = tile - zy * strips;
+        const int cc = min(c, ncols - 1);
+        const int tile = cc / BN, r = cc - tile * BN;
+        int zy, strip;
+        strip_of_tile(tile, imgrow_div, img_rows, zy, strip);
+        zy = __builtin_amdgcn_readfirstlane(zy);
         const int z = (int)h_div.div((unsigned)zy);
         const int y = zy - z * H;
         const int pix = r / N, nn = r - pix * N;
+        const int x = strip * OUT_PIX + pad_w - 2 + pix;
         Col o;
-        o.z0 = z + pad_d; o.y0 = y + pad_h; o.x0 = strip * OUT_PIX + pad_w - 2 + pix;
-        o.base = ((o.z0 * P + o.y0) * Q + o.x0) * N + nn;
+        o.z0 = z + pad_d; o.y0 = y + pad_h;
+        o.xok = (c < ncols) & ((unsigned)x < (unsigned)Q);
+        o.base = (unsigned)(((o.z0 * P + o.y0) * Q + x) * N + nn) * (unsigned)sizeof(T);
         return o;
     }
-    __device__ __forceinline__ unsigned offset(const Fixed& f, const Col& c) const
+    // kr: row inside the tile (uniform over the wavefront)
+    __device__ __forceinline__ unsigned offset(const Fixed& f, int kr, const Col& c) const
     {
-        return stream_offset<T>(f, c, M, P, Q);
+        const bool rowok = ((unsigned)(c.z0 + f.dz) < (unsigned)M) & ((unsigned)(c.y0 + f.dy) < (unsigned)P) & (kr < f.kleft);
+        return (rowok & c.xok) ? c.base + (unsigned)(f.off + kr * row_stride * (int)sizeof(T)) : NG_OOB_OFFSET;
     }
 };
 

@@ -35,6 +35,13 @@ __device__ __forceinline__ void static_for(F&& f)
     }
 }
 
+// A gather whose contraction rows differ only by a uniform stride inside a tile
+// declares `static constexpr bool FIXED_PER_TILE = true`, Fixed fixed(first row of
+// the tile) and offset(Fixed, row inside the tile, Col): one Fixed per contraction
+// tile is kept (in scalar registers) instead of one per request.
+template <class G, class = void> struct GatherFixedPerTile { static constexpr bool value = false; };
+template <class G> struct GatherFixedPerTile<G, std::enable_if_t<G::FIXED_PER_TILE>> { static constexpr bool value = true; };
+
 template <class E, class = void> struct StoresPerThread { static constexpr int value = 0; };
 template <class E> struct StoresPerThread<E, std::enable_if_t<(E::STORES_PER_THREAD > 0)>> { static constexpr int value = E::STORES_PER_THREAD; };
 
@@ -109,7 +116,10 @@ void mfma_stream_kernel(ALoad aload, BGather bg, Epi epi, int tiles)
     static_assert(!WHOLE || BM == 32, "whole-tile epilogues take one block of 32 rows");
     constexpr int EPITCH = WTN * 4 + 16;
     constexpr int EPI_BYTES = 32 * EPITCH;
-    constexpr int EPI_REGION = WHOLE ? EpilogueStagedRows<Epi>::value * BN * 4 : EPI_BYTES * WN;
+    // a whole-tile epilogue parks its rows in the ring stage that was just multiplied
+    // (free until the request behind the next barrier), so it needs no LDS of its own
+    constexpr int EPI_REGION = WHOLE ? 0 : EPI_BYTES * WN;
+    static_assert(!WHOLE || EpilogueStagedRows<Epi>::value * BN * 4 <= TB::BYTES, "parked rows must fit one ring stage");
     constexpr int RING = NSTAGE * TB::BYTES;
     static_assert(RING + EPI_REGION <= 160 * 1024, "ring and epilogue staging exceed the LDS of a compute unit");
     __shared__ __attribute__((aligned(16))) char smem[RING + EPI_REGION];
@@ -152,14 +162,23 @@ void mfma_stream_kernel(ALoad aload, BGather bg, Epi epi, int tiles)
     }
 
     // ---- B stream ----
-    int rc[CPT_B];
-    typename BGather::Fixed fx[KT][CPT_B];
+    constexpr bool PER_TILE = GatherFixedPerTile<BGather>::value;
+    static_assert(!PER_TILE || TB::CPR == 64, "a tile line must be one wavefront request for its row to be uniform");
+    int rc[CPT_B], kc[CPT_B];
+    typename BGather::Fixed fx[KT][PER_TILE ? 1 : CPT_B];
 #pragma unroll
     for (int c = 0; c < CPT_B; c++) {
         int k;
         TB::chunk_pos(tid + c * NT, rc[c], k);
+        kc[c] = PER_TILE ? __builtin_amdgcn_readfirstlane(k) : k;
+        if constexpr (!PER_TILE) {
 #pragma unroll
-        for (int kt = 0; kt < KT; kt++) fx[kt][c] = bg.fixed(kt * BK + k);
+            for (int kt = 0; kt < KT; kt++) fx[kt][c] = bg.fixed(kt * BK + k);
+        }
+    }
+    if constexpr (PER_TILE) {
+#pragma unroll
+        for (int kt = 0; kt < KT; kt++) fx[kt][0] = bg.fixed(kt * BK);
     }
     const BufferRsrc rsrc = make_rsrc(bg.X);
     typename BGather::Col col[CPT_B];
@@ -176,7 +195,10 @@ void mfma_stream_kernel(ALoad aload, BGather bg, Epi epi, int tiles)
                 unsigned off = NG_OOB_OFFSET;
 #pragma unroll
                 for (int q = 0; q < KT; q++)
-                    if (q == ktn) off = bg.offset(fx[q][c], col[c]);
+                    if (q == ktn) {
+                        if constexpr (PER_TILE) off = bg.offset(fx[q][0], kc[c], col[c]);
+                        else                    off = bg.offset(fx[q][c], col[c]);
+                    }
                 buffer_load_chunk_to_lds(rsrc, smem + wr_off + (c * NT + wave * 64) * 16, off);
             }
         }
@@ -226,7 +248,8 @@ void mfma_stream_kernel(ALoad aload, BGather bg, Epi epi, int tiles)
             __syncthreads();
             // behind the barrier nobody reads the stage of tile q-1 any more
             issue(i + (kt + D) / KT, (kt + D) % KT);
-            const char* tile = smem + rd_off;
+            const int stage_off = rd_off;
+            const char* tile = smem + stage_off;
 #pragma unroll
             for (int st = 0; st < KS; st++) {
                 Frag<T> fb[TN];
@@ -241,8 +264,9 @@ void mfma_stream_kernel(ALoad aload, BGather bg, Epi epi, int tiles)
             if (kt == KT - 1) {
                 const int n0 = (first + i) * BN;
                 if constexpr (WHOLE) {
-                    float* g = reinterpret_cast<float*>(smem + RING);
+                    float* g = reinterpret_cast<float*>(smem + stage_off);
                     const int nrows = epi.rows;
+                    __syncthreads();   // every wavefront is done with the fragments of this stage
 #pragma unroll
                     for (int j = 0; j < TN; j++)
 #pragma unroll
@@ -252,9 +276,8 @@ void mfma_stream_kernel(ALoad aload, BGather bg, Epi epi, int tiles)
                         }
                     __syncthreads();
                     epi.tile_buffer(out_rsrc, g, tid, n0);
-                    // the next column tile parks its rows only after KT more barriers;
-                    // with a single contraction tile that is the very next one
-                    if (KT == 1) __syncthreads();
+                    // the stage is requested into again behind the next barrier, which every
+                    // thread reaches only after it has read the parked rows
                 } else {
                     StreamBands<TM, TN, WTN, EPITCH, 0>::run(acc, smem + RING + wave * EPI_BYTES, lane, n0 + wave * WTN, out_rsrc, epi);
                 }
