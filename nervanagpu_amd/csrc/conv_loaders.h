@@ -297,44 +297,58 @@ struct GatherRowSegLoader {
     static constexpr bool DIRECT = true;
     static constexpr bool TILE_READS_TABLE = false;
 
-    struct Ctx { int base, z0, y0, kr; };
-    struct Tile { BufferRsrc rsrc; int toff, dz, dy, k0; };
+    // The image row (z, y) of a tile is the same for all its chunks and the filter
+    // row of a contraction tile is uniform anyway, so the row test runs on the
+    // scalar unit; per lane remain one add and one select.  The channel count is a
+    // multiple of BK (the host checks), so no chunk lies past the last channel.
+    struct Ctx { unsigned base; int z0, y0; bool xok; };
+    struct Tile { BufferRsrc rsrc; int toff, dz, dy; int blk, ft, fr; };
     typedef NoWaveState Wave;
     __device__ __forceinline__ Wave wave_init(int /*lane*/) const { return Wave{}; }
 
     __device__ __forceinline__ Ctx prepare_seg(int n0, int r, int kr) const
     {
         Ctx c;
-        c.kr = kr;
-        c.base = 0; c.z0 = c.y0 = NG_FAR;
-        if (n0 >= lat.ncols) return c;
         int iz, iy, ix0, nn0;
-        lat.split(n0, iz, iy, ix0, nn0);
+        lat.split(min(n0, lat.ncols - 1), iz, iy, ix0, nn0);
         const int pix = r / TAP_COLS, nn = r - pix * TAP_COLS;
         const int ix = ix0 + pix - pad_w;
-        if ((unsigned)ix >= (unsigned)W) return c;
-        c.z0 = iz; c.y0 = iy;
-        c.base = ((iz * H + iy) * W + ix) * lat.N + nn + kr * row_stride;
+        c.xok = (n0 < lat.ncols) & ((unsigned)ix < (unsigned)W);
+        c.z0 = __builtin_amdgcn_readfirstlane(iz);
+        c.y0 = __builtin_amdgcn_readfirstlane(iy);
+        c.base = (unsigned)(((iz * H + iy) * W + ix) * lat.N + nn + kr * row_stride) * (unsigned)sizeof(T);
         return c;
+    }
+    __device__ __forceinline__ void place(Tile& t) const
+    {
+        t.dz = t.ft - pad_d; t.dy = t.fr - pad_h;
+        t.toff = ((t.dz * H + t.dy) * W * lat.N + t.blk * BK * row_stride) * (int)sizeof(T);
     }
     __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/, const Wave&) const
     {
         Tile t;
         t.rsrc = make_rsrc(X);
-        const int blk = (int)tr_div.div((unsigned)kt);
-        const int tr = kt - blk * TR;
-        const int ft = (int)r_div.div((unsigned)tr);
-        const int fr = tr - ft * R;
-        t.dz = ft - pad_d; t.dy = fr - pad_h;
-        t.toff = (t.dz * H + t.dy) * W * lat.N + blk * BK * row_stride;
-        t.k0 = chan - blk * BK;
+        t.blk = (int)tr_div.div((unsigned)kt);
+        const int tr = kt - t.blk * TR;
+        t.ft = (int)r_div.div((unsigned)tr);
+        t.fr = tr - t.ft * R;
+        place(t);
         return t;
+    }
+    // next contraction tile: filter rows (t, r) are the fast index, channel blocks the slow one
+    static constexpr bool INCREMENTAL = true;
+    __device__ __forceinline__ void advance(Tile& t, int /*bk*/) const
+    {
+        if (++t.fr == R) {
+            t.fr = 0;
+            if (++t.ft * R == TR) { t.ft = 0; t.blk++; }
+        }
+        place(t);
     }
     __device__ __forceinline__ unsigned offset(const Tile& t, const Ctx& c) const
     {
-        const bool ok = ((unsigned)(c.z0 + t.dz) < (unsigned)D) & ((unsigned)(c.y0 + t.dy) < (unsigned)H) & (c.kr < t.k0);
-        const unsigned off = (unsigned)(c.base + t.toff) * (unsigned)sizeof(T);
-        return ok ? off : NG_OOB_OFFSET;
+        const bool rowok = ((unsigned)(c.z0 + t.dz) < (unsigned)D) & ((unsigned)(c.y0 + t.dy) < (unsigned)H);
+        return (rowok & c.xok) ? c.base + (unsigned)t.toff : NG_OOB_OFFSET;
     }
     __device__ __forceinline__ uint4_t load(const Tile& t, const Ctx& c) const { return buffer_load_chunk(t.rsrc, offset(t, c)); }
 };
@@ -354,7 +368,7 @@ struct FilterTapRowLoader {
     static constexpr bool TILE_READS_TABLE = false;
 
     struct Ctx { unsigned off; int c; };
-    struct Tile { BufferRsrc rsrc; int rows; };
+    struct Tile { BufferRsrc rsrc; const T* p; int rows, tr; };
     typedef NoWaveState Wave;
     __device__ __forceinline__ Wave wave_init(int /*lane*/) const { return Wave{}; }
 
@@ -369,11 +383,24 @@ struct FilterTapRowLoader {
     __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/, const Wave&) const
     {
         const int blk = (int)tr_div.div((unsigned)kt);
-        const int tr = kt - blk * TR;
         Tile t;
-        t.rsrc = make_rsrc(F + (long)blk * BK * RSTK + (long)tr * TAPS * K);
+        t.tr = kt - blk * TR;
+        t.p = F + (long)blk * BK * RSTK + (long)t.tr * TAPS * K;
+        t.rsrc = make_rsrc(t.p);
         t.rows = C - blk * BK;
         return t;
+    }
+    // next contraction tile: the next filter row, or the first one of the next channel block
+    static constexpr bool INCREMENTAL = true;
+    __device__ __forceinline__ void advance(Tile& t, int /*bk*/) const
+    {
+        t.p += TAPS * K;
+        if (++t.tr == TR) {
+            t.tr = 0;
+            t.p += (long)BK * RSTK - (long)TR * TAPS * K;
+            t.rows -= BK;
+        }
+        t.rsrc = make_rsrc(t.p);
     }
     __device__ __forceinline__ unsigned offset(const Tile& t, const Ctx& c) const
     {
@@ -401,7 +428,7 @@ struct FilterTapColsLoader {
     static constexpr bool TILE_READS_TABLE = false;
 
     struct Ctx { unsigned off; int kc; };
-    struct Tile { BufferRsrc rsrc; int kvalid; };
+    struct Tile { BufferRsrc rsrc; const T* p; int kvalid, tr; };
     typedef NoWaveState Wave;
     __device__ __forceinline__ Wave wave_init(int /*lane*/) const { return Wave{}; }
 
@@ -413,17 +440,28 @@ struct FilterTapColsLoader {
         c.off = (m < C) ? (unsigned)(m * RSTK + (TAPS - 1 - tap) * K + c.kc) * (unsigned)sizeof(T) : NG_OOB_OFFSET;
         return c;
     }
+    // tile (block, t', r') reads filter row TR-1 - (t'*R + r') (both coordinates mirrored)
     __device__ __forceinline__ Tile tile(int kt, int /*k0*/, int /*zb*/, const Wave&) const
     {
         const int blk = (int)tr_div.div((unsigned)kt);
-        const int tr = kt - blk * TR;
-        const int ft = (int)r_div.div((unsigned)tr);
-        const int fr = tr - ft * R;
-        const int row = (TR / R - 1 - ft) * R + (R - 1 - fr);
         Tile t;
-        t.rsrc = make_rsrc(F + (long)row * TAPS * K + (long)blk * BK);
+        t.tr = kt - blk * TR;
+        t.p = F + (long)(TR - 1 - t.tr) * TAPS * K + (long)blk * BK;
+        t.rsrc = make_rsrc(t.p);
         t.kvalid = K - blk * BK;
         return t;
+    }
+    // next contraction tile: the filter row before, or the last one for the next block of output maps
+    static constexpr bool INCREMENTAL = true;
+    __device__ __forceinline__ void advance(Tile& t, int /*bk*/) const
+    {
+        t.p -= TAPS * K;
+        if (++t.tr == TR) {
+            t.tr = 0;
+            t.p += (long)TR * TAPS * K + BK;
+            t.kvalid -= BK;
+        }
+        t.rsrc = make_rsrc(t.p);
     }
     // K is a multiple of the chunk length, so a chunk is inside or outside as a whole
     __device__ __forceinline__ unsigned offset(const Tile& t, const Ctx& c) const
