@@ -379,6 +379,10 @@ __device__ __forceinline__ void wave_lds_fence()
     __builtin_amdgcn_wave_barrier();
 }
 
+// epilogues with a descriptor-store form of their plain case declare BUFFER_STORE
+template <class E, class = void> struct EpilogueBufferStore { static constexpr bool value = false; };
+template <class E> struct EpilogueBufferStore<E, std::enable_if_t<E::BUFFER_STORE>> { static constexpr bool value = true; };
+
 template <int TM, int TN, int WTN, int EPITCH, int I>
 struct EpilogueBands {
     template <class Epi>
@@ -395,15 +399,37 @@ struct EpilogueBands {
                 *reinterpret_cast<float*>(stage + ((v >> 2) * 8 + rsub + (v & 3)) * EPITCH + (j * 32 + col) * 4) =
                     acc[I][j][v];
         wave_lds_fence();
+        // The common store (16-bit output, aligned rows, no beta, nearest rounding,
+        // no mask) goes through a buffer descriptor: edges are dropped by the
+        // hardware and the address is a 32-bit offset, a third of the instructions
+        // of the general store8 with its run-time choices.
+        bool plain = false;
+        if constexpr (EpilogueBufferStore<Epi>::value) plain = epi.plain_store();
+        if (plain) {
+            if constexpr (EpilogueBufferStore<Epi>::value) {
+                const BufferRsrc rsrc = epi.store_rsrc(z);
 #pragma unroll
-        for (int c = 0; c < CPW / 64; c++) {
-            const int id = lane + c * 64;
-            const int r = id / (WTN / 8);
-            const int cc = (id % (WTN / 8)) * 8;
-            const float4_t lo = *reinterpret_cast<const float4_t*>(stage + r * EPITCH + cc * 4);
-            const float4_t hi = *reinterpret_cast<const float4_t*>(stage + r * EPITCH + cc * 4 + 16);
-            const float vals[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            epi.store8(mbase + I * 32 + r, nbase + cc, z, split, vals);
+                for (int c = 0; c < CPW / 64; c++) {
+                    const int id = lane + c * 64;
+                    const int r = id / (WTN / 8);
+                    const int cc = (id % (WTN / 8)) * 8;
+                    const float4_t lo = *reinterpret_cast<const float4_t*>(stage + r * EPITCH + cc * 4);
+                    const float4_t hi = *reinterpret_cast<const float4_t*>(stage + r * EPITCH + cc * 4 + 16);
+                    const float vals[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    epi.store8_buffer(rsrc, mbase + I * 32 + r, nbase + cc, vals);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < CPW / 64; c++) {
+                const int id = lane + c * 64;
+                const int r = id / (WTN / 8);
+                const int cc = (id % (WTN / 8)) * 8;
+                const float4_t lo = *reinterpret_cast<const float4_t*>(stage + r * EPITCH + cc * 4);
+                const float4_t hi = *reinterpret_cast<const float4_t*>(stage + r * EPITCH + cc * 4 + 16);
+                const float vals[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                epi.store8(mbase + I * 32 + r, nbase + cc, z, split, vals);
+            }
         }
         wave_lds_fence();
         if constexpr (I + 1 < TM)
@@ -1078,6 +1104,13 @@ struct ScaleStoreEpilogue {
     FastDiv  fold_div = FastDiv{0, 0};
 
     __device__ __forceinline__ const void* base() const { return C; }
+    static constexpr bool BUFFER_STORE = sizeof(bits_t) == 2;
+    // the case store8_buffer covers (uniform over the launch)
+    __device__ __forceinline__ bool plain_store() const
+    {
+        return vec && beta == 0.0f && sr_bits == 0u && mask == nullptr && fold_from == 0 && (long)m * ldc < (1L << 30);
+    }
+    __device__ __forceinline__ BufferRsrc store_rsrc(int z) const { return make_rsrc(C + (long)z * ldcz); }
     __device__ __forceinline__ bool masked_out(long offset) const
     {
         return !(StoreBits<T>::widen(reinterpret_cast<const bits_t*>(mask)[offset]) > 0.0f);
@@ -1117,7 +1150,6 @@ struct ScaleStoreEpilogue {
     // outside the matrix are dropped by the hardware instead of branched around.
     __device__ __forceinline__ void store8_buffer(BufferRsrc rsrc, int i, int j0, const float (&acc)[8]) const
     {
-        static_assert(sizeof(bits_t) == 2, "descriptor stores are written for 16-bit outputs");
         bits_t out[8];
         if (relu) {
 #pragma unroll
@@ -1126,8 +1158,10 @@ struct ScaleStoreEpilogue {
 #pragma unroll
             for (int e = 0; e < 8; e++) out[e] = StoreBits<T>::round(acc[e] * alpha, 0, 0, 0, 0);
         }
-        const unsigned off = (i < m && j0 < n) ? ((unsigned)i * (unsigned)ldc + (unsigned)j0) * 2u : NG_OOB_OFFSET;
-        buffer_store_chunk(rsrc, off, *reinterpret_cast<const uint4_t*>(out));
+        if constexpr (sizeof(bits_t) == 2) {
+            const unsigned off = (i < m && j0 < n) ? ((unsigned)i * (unsigned)ldc + (unsigned)j0) * 2u : NG_OOB_OFFSET;
+            buffer_store_chunk(rsrc, off, *reinterpret_cast<const uint4_t*>(out));
+        }
     }
     __device__ __forceinline__ void store8(int i, int j0, int z, int /*split*/, const float (&acc)[8]) const
     {
