@@ -146,12 +146,13 @@ static bool shares_taps(const ConvPlan& pl)
            p.str_d == 1 && p.str_h == 1 && p.str_w == 1 && !pl.merged;
 }
 
-template <int BM, int WM, int WN>
+template <int BM, int WM, int WN, int BN = 256>
 static int bprop_shared_taps(const ConvPlan& pl, const void* F, const void* E, void* gradI, float alpha,
-                             const void* mask, hipStream_t stream)
+                             const void* mask, hipStream_t stream, int col_begin = 0, int col_end = -1)
 {
     typedef _Float16 T;
-    constexpr int BN = 256, BK = 32, TAPS = 3, COLS = 64;
+    constexpr int BK = 32, TAPS = 3, COLS = 64;
+    static_assert(BN == 4 * COLS || BN == COLS, "four pixels per tile, or one (tail launch)");
     const ng_conv_params& p = pl.p;
     const int ncols = p.D * p.H * p.W * p.N;
     const int TR = p.T * p.R, nblk = cdiv(p.K, BK);
@@ -162,7 +163,8 @@ static int bprop_shared_taps(const ConvPlan& pl, const void* F, const void* E, v
                                              p.T - 1 - p.pad_d, p.R - 1 - p.pad_h, p.S - 1 - p.pad_w,
                                              p.M * p.P * p.Q * p.N,
                                              FastDiv::make((unsigned)TR), FastDiv::make((unsigned)p.R), TR, p.R, p.K};
-    return launch_core<T, BM, BN, BK, WM, WN, KC, MC>(al, bl, epi, p.C, ncols, TR * nblk, 1, stream, "conv bprop (shared taps)");
+    return launch_core<T, BM, BN, BK, WM, WN, KC, MC>(al, bl, epi, p.C, ncols, TR * nblk, 1, stream, "conv bprop (shared taps)",
+                                                      col_begin, col_end);
 }
 
 // Very few channels (a first layer): rows (channel, horizontal tap), see
@@ -256,7 +258,17 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
     if constexpr (sizeof(T) == 2) {
         if (thin_channels(pl, mask)) return bprop_thin(pl, F, E, gradI, alpha, stream);
         if (shares_taps(pl)) {
-            switch (pick_row_tile(p.C, p.D * p.H * p.W * p.N, 256)) {
+            const int ncols = p.D * p.H * p.W * p.N;
+            const int row_tile = pick_row_tile(p.C, ncols, 256);
+            // trailing column tiles beyond whole rounds: 64x64 tiles behind the main launch
+            const int tail = row_tile >= 128 ? tail_column_tiles(cdiv(p.C, row_tile), cdiv(ncols, 256)) : 0;
+            if (tail) {
+                const int cut = (cdiv(ncols, 256) - tail) * 256;
+                const int rc = row_tile == 256 ? bprop_shared_taps<256, 2, 4>(pl, F, E, gradI, alpha, mask, stream, 0, cut)
+                                               : bprop_shared_taps<128, 2, 4>(pl, F, E, gradI, alpha, mask, stream, 0, cut);
+                return rc ? rc : bprop_shared_taps<64, 2, 2, 64>(pl, F, E, gradI, alpha, mask, stream, cut, -1);
+            }
+            switch (row_tile) {
             case 256: return bprop_shared_taps<256, 2, 4>(pl, F, E, gradI, alpha, mask, stream);
             case 128: return bprop_shared_taps<128, 2, 4>(pl, F, E, gradI, alpha, mask, stream);
             default:  return bprop_shared_taps<64, 1, 4>(pl, F, E, gradI, alpha, mask, stream);

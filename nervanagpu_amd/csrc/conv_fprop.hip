@@ -43,14 +43,16 @@ static bool shares_taps(const ConvPlan& pl)
            p.str_d == 1 && p.str_h == 1 && p.str_w == 1;
 }
 
-// COLS = N images per pixel; a tile of BN = 4 * COLS columns is four output pixels
+// COLS = N images per pixel; a tile of BN columns is BN / COLS output pixels of one
+// image row (four, or one for the 64-column tiles of a tail launch); the image rows are
+// padded to a multiple of four pixels
 template <int BM, int WM, int WN, int BN = 256, int COLS = 64>
 static int fprop_shared_taps(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags,
-                             hipStream_t stream)
+                             hipStream_t stream, int col_begin = 0, int col_end = -1)
 {
     typedef _Float16 T;
     constexpr int BK = 32, TAPS = 3;
-    static_assert(BN == 4 * COLS, "four output pixels per tile");
+    static_assert(BN == 4 * COLS || BN == COLS, "four output pixels per tile, or one");
     const ng_conv_params& p = pl.p;
     const int qpad = cdiv(p.Q, 4) * 4;
     const int ncols = p.M * p.P * qpad * p.N;           // the kernel's columns: padded image rows
@@ -65,7 +67,8 @@ static int fprop_shared_taps(const ConvPlan& pl, const void* I, const void* F, v
     GatherRowSegLoader<T, BK, TAPS, COLS> bl{(const T*)I, PixelLattice::make(p.N, ncols, qpad, p.P * qpad), p.D, p.H, p.W,
                                              p.pad_d, p.pad_h, p.pad_w, p.D * p.H * p.W * p.N,
                                              FastDiv::make((unsigned)TR), FastDiv::make((unsigned)p.R), TR, p.R, p.C};
-    return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, epi, p.K, ncols, TR * nblk, 1, stream, "conv fprop (shared taps)");
+    return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, epi, p.K, ncols, TR * nblk, 1, stream, "conv fprop (shared taps)",
+                                                      col_begin, col_end);
 }
 
 // A filter of at most 64 output maps and 128 contraction rows (a first layer on
@@ -105,7 +108,18 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
             // 32 images: 128-column tiles; 128 rows on four wavefronts
             if (pl.p.K >= 128) return fprop_shared_taps<128, 2, 2, 128, 32>(pl, I, F, O, alpha, flags, st);
         } else if (shares_taps(pl)) {
-            switch (pick_row_tile(pl.p.K, pl.p.M * pl.p.P * cdiv(pl.p.Q, 4) * 4 * pl.p.N, 256)) {
+            const int ncols = pl.p.M * pl.p.P * cdiv(pl.p.Q, 4) * 4 * pl.p.N;
+            const int row_tile = pick_row_tile(pl.p.K, ncols, 256);
+            // the few column tiles beyond whole rounds of one-per-CU workgroups run
+            // behind the main launch as 64x64 tiles, which cover the chip at once
+            const int tail = row_tile >= 128 ? tail_column_tiles(cdiv(pl.p.K, row_tile), cdiv(ncols, 256)) : 0;
+            if (tail) {
+                const int cut = (cdiv(ncols, 256) - tail) * 256;
+                const int rc = row_tile == 256 ? fprop_shared_taps<256, 2, 4>(pl, I, F, O, alpha, flags, st, 0, cut)
+                                               : fprop_shared_taps<128, 2, 4>(pl, I, F, O, alpha, flags, st, 0, cut);
+                return rc ? rc : fprop_shared_taps<64, 2, 2, 64, 64>(pl, I, F, O, alpha, flags, st, cut, -1);
+            }
+            switch (row_tile) {
             case 256: return fprop_shared_taps<256, 2, 4>(pl, I, F, O, alpha, flags, st);
             case 128: return fprop_shared_taps<128, 2, 4>(pl, I, F, O, alpha, flags, st);
             default:  return fprop_shared_taps<64, 1, 4>(pl, I, F, O, alpha, flags, st);

@@ -109,16 +109,33 @@ inline int pick_row_tile(int rows, int ncols, int bn)
     return best;
 }
 
+// A grid of one-per-CU workgroups that is a few tiles more than a whole number
+// of rounds over the chip spends a full round on those few (784 tiles on 256 CUs:
+// four rounds for 3.06).  Returns how many trailing column tiles to take out of
+// the main launch and run behind it as many small tiles that cover the chip at
+// once: the remainder, when there is a single row tile, at least one full round,
+// and the remainder is at most a quarter of the chip; else 0.
+inline int tail_column_tiles(int tiles_m, int tiles_n)
+{
+    const int cus = device_cu_count();
+    if (tiles_m != 1 || tiles_n <= cus) return 0;
+    const int rem = tiles_n % cus;
+    return (rem > 0 && 4 * rem <= cus) ? rem : 0;
+}
+
+// col_begin / col_end: the column range this launch covers (multiples of BN; default: all)
 template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, int NSTAGE = 2, class AL, class BL, class Epi>
 inline int launch_core(const AL& al, const BL& bl, const Epi& epi, int rows, int ncols, int k_tiles, int splits,
-                       hipStream_t stream, const char* what)
+                       hipStream_t stream, const char* what, int col_begin = 0, int col_end = -1)
 {
+    if (col_end < 0) col_end = ncols;
     CoreShape s;
     s.m = rows; s.n = ncols;
     s.k_tiles = k_tiles;
     s.passes = 1; s.splits = splits;
     s.tiles_m = cdiv(rows, BM);
-    s.tiles_n = cdiv(ncols, BN);
+    s.tiles_n = cdiv(col_end - col_begin, BN);
+    s.n_base = col_begin;
     launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB, NSTAGE>(dim3(grid_tiles(s.tiles_m * s.tiles_n, splits), grid_slices(s.tiles_m * s.tiles_n, splits), 1), stream, al, bl, epi, s);
     NG_CHECK_LAUNCH(what);
     return 0;

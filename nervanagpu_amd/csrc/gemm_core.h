@@ -141,6 +141,7 @@ struct CoreShape {
     int passes;        // contraction passes accumulated into one output (batch_loops)
     int splits;        // the (passes * k_tiles) tile range is cut into this many slices
     int tiles_m, tiles_n;
+    int n_base = 0;    // first column of this launch's tile 0 (a launch may cover a column range of the problem)
 };
 
 // gridDim.y of a launch over `tiles` output tiles (gridDim.x) and `splits`
@@ -467,7 +468,7 @@ void mfma_gemm_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
 
     int tm, tn, split;
     if (!block_work(s, tm, tn, split)) return;
-    const int m0 = tm * BM, n0 = tn * BN;
+    const int m0 = tm * BM, n0 = s.n_base + tn * BN;
     const int z = blockIdx.z;
 
     // contraction tile range of this split
@@ -801,7 +802,7 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
 
     int tm, tn, split;
     if (!block_work(s, tm, tn, split)) return;
-    const int m0 = tm * BM, n0 = tn * BN;
+    const int m0 = tm * BM, n0 = s.n_base + tn * BN;
     const int z = blockIdx.z;
 
     const int total_tiles = s.passes * s.k_tiles;

@@ -62,6 +62,10 @@ SMALL = [
     (16, 3, 8, 1, 70, 70, 1, 6, 6, (0, 2, 2), (1, 1, 1)),
     (64, 3, 64, 1, 20, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     (64, 5, 32, 1, 24, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    # 288 column tiles of 256 on a 256-CU chip: the 32 tiles beyond a whole round run as 64x64 tiles in a
+    # second launch (forward with 128 output maps; data gradient with 128 channels)
+    (64, 32, 128, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (64, 128, 32, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     # long pixel ranges with filter rows in multiples of 192: the weight gradient's 192-row tiles
     (64, 64, 32, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     (64, 64, 96, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
@@ -70,7 +74,8 @@ SMALL = [
 
 # cases that exist for a half-precision kernel and are large
 FP16_ONLY = {(64, 3, 64, 1, 20, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 5, 32, 1, 24, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
-             (32, 32, 128, 2, 5, 8, 2, 3, 3, (1, 1, 1), (1, 1, 1)), (32, 64, 136, 1, 6, 12, 1, 3, 3, (0, 1, 1), (1, 1, 1))}
+             (32, 32, 128, 2, 5, 8, 2, 3, 3, (1, 1, 1), (1, 1, 1)), (32, 64, 136, 1, 6, 12, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+             (64, 32, 128, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 128, 32, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1))}
 
 
 def _layer(ng, dtype, case):
@@ -343,8 +348,13 @@ def test_bprop_with_rectifier_mask(ng, dtype):
     relu derivative step `grad *= act > 0` (nervanagpu/layers.py:89-91), on the
     blocked, the row-by-row and the shared-tap form, full and ragged tiles; strided layers refuse."""
     rng = np.random.default_rng(29)
-    for case in (SMALL[0], SMALL[2], SMALL[5], SMALL[8], SMALL[11], SMALL[21], SMALL[23],
-                 (16, 64, 64, 1, 20, 20, 1, 3, 3, (0, 1, 1), (1, 1, 1))):
+    for case in (SMALL[0], SMALL[2], SMALL[5], SMALL[8], SMALL[11],
+                 (64, 72, 96, 1, 5, 12, 1, 3, 3, (0, 0, 0), (1, 1, 1)),        # shared taps
+                 (64, 32, 64, 3, 4, 8, 3, 2, 3, (2, 0, 1), (1, 1, 1)),         # shared taps, 3-D
+                 (16, 64, 64, 1, 20, 20, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+                 (64, 128, 32, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1))):     # main launch + tail launch
+        if dtype == np.float32 and case in FP16_ONLY:
+            continue
         layer = _layer(ng, dtype, case)
         I, F, E = _data(layer, dtype, 31)
         act = np.maximum(rng.standard_normal(layer.dimI), 0).astype(dtype)     # about half zeros
