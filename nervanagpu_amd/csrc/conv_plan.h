@@ -54,25 +54,33 @@ inline int cdiv(int a, int b) { return (a + b - 1) / b; }
 // channel blocks of depth bk: exact, or padded by at most one half
 inline bool blocks_pay(int channels, int bk) { return channels % bk == 0 || 2 * cdiv(channels, bk) * bk <= 3 * channels; }
 
-// how many slices to cut a contraction into so that the grid fills the chip:
-// one and a half workgroups per CU when every slice still keeps 30 or more
-// tiles (measured 10-35 % faster weight gradients at AlexNet / VGG sizes: a
-// second workgroup on half of the CUs overlaps the tile-step latency of the
-// first), one per CU for short contractions, where the extra fp32 partials
-// cost more than the overlap gains
-// (`halves`: workgroups per CU in halves; the 64x64 tile of the smallest
-// filters needs a fifth of the LDS and gains from three per CU: VGG conv1
-// weight gradient 119 -> 86 us)
-inline int conv_splits(int out_tiles, int total_k_tiles, size_t slice_bytes, size_t ws_bytes, int halves = 3)
+// how many slices to cut a contraction into: as many as fill every workgroup
+// slot of the chip exactly once (`per_cu` workgroups of this tile shape fit the
+// LDS of a CU), rounded down.  Workgroups that share a CU share its matrix
+// pipes, so a grid is as slow as its fullest CU: one and a half workgroups per
+// CU cost what two cost, and a grid a few workgroups over a whole round costs a
+// round more (VGG weight gradients 7-22 % faster than with a rounded-up one and
+// a half per CU).  Contractions too short to leave 15 tiles per slice get one
+// workgroup per CU: the fp32 partials then cost more than the overlap gains.
+inline int conv_splits(int out_tiles, int total_k_tiles, size_t slice_bytes, size_t ws_bytes, int per_cu = 2)
 {
     const int cus = device_cu_count();
-    if (out_tiles >= cus || total_k_tiles < 8) return 1;
-    int splits = cdiv(halves * cus / 2, out_tiles);
-    if (total_k_tiles / splits < 30) splits = cdiv(cus, out_tiles);
-    splits = std::min(splits, total_k_tiles / 4);
+    if (total_k_tiles < 8) return 1;
+    int splits = std::max(1, cus * per_cu / out_tiles);
+    if (total_k_tiles / splits < 15) splits = std::max(1, cus / out_tiles);
+    splits = std::min(splits, std::max(1, total_k_tiles / 4));
     if (slice_bytes) splits = (int)std::min<size_t>((size_t)splits, ws_bytes / slice_bytes);
     while (splits > 1 && (splits - 1) * cdiv(total_k_tiles, splits) >= total_k_tiles) splits--;
     return std::max(splits, 1);
+}
+
+// workgroups of a weight-gradient tile shape (64-deep, two stages) that fit
+// the LDS of a CU: three of the 64x64 tile (measured better than four: VGG
+// conv1 119 -> 86 us against two), one of 256x256, two of the shapes between
+inline int update_tiles_per_cu(int bm, int bn)
+{
+    if (bm == 64 && bn == 64) return 3;
+    return bm >= 256 ? 1 : 2;
 }
 
 inline int check_ptr16(const void* p, const char* what)

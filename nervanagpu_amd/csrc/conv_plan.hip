@@ -143,10 +143,10 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
     {
         const int kt = cdiv(p.M * p.P * p.Q * p.N, pl->bk);
         // the most slices any tile shape of the update dispatcher would ask for
-        int splits = std::max(conv_splits(cdiv(pl->CRST, 128) * cdiv(p.K, 128), kt, 0, 0),
-                              conv_splits(cdiv(pl->CRST, 256) * cdiv(p.K, 256), kt, 0, 0));
-        if (p.K <= 64 && pl->CRST <= 64) splits = std::max(splits, conv_splits(1, kt, 0, 0, 6));
-        splits = std::max(splits, conv_splits(cdiv(pl->CRST, 192) * cdiv(p.K, p.K <= 64 ? 64 : 128), kt, 0, 0));
+        static const int shapes[6][2] = {{128, 128}, {256, 256}, {64, 64}, {192, 64}, {192, 128}, {128, 64}};
+        int splits = 1;
+        for (const auto& t : shapes)
+            splits = std::max(splits, conv_splits(cdiv(pl->CRST, t[0]) * cdiv(p.K, t[1]), kt, 0, 0, update_tiles_per_cu(t[0], t[1])));
         pl->ws_update = splits > 1 ? align_up((size_t)splits * pl->CRST * p.K * sizeof(float), 256) : 0;
     }
     *plan_out = pl;

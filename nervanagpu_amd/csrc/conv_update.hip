@@ -17,7 +17,7 @@ static int launch_update(const ConvPlan& pl, const void* I, const void* E, void*
     const int k_tiles = cdiv(kdim, BK);
     const int tiles = cdiv(rows, BM) * cdiv(cols, BN);
     const size_t slice = (size_t)rows * cols * sizeof(float);
-    const int splits = ws ? conv_splits(tiles, k_tiles, slice, ws_bytes, (BM == 64 && BN == 64) ? 6 : 3) : 1;
+    const int splits = ws ? conv_splits(tiles, k_tiles, slice, ws_bytes, update_tiles_per_cu(BM, BN)) : 1;
     const int npt = BLOCKED ? p.N / BK : 1;
 
     GatherRowsLoader<T, TIN, BLOCKED, BK> al{(const TIN*)I, pl.d_fprop_flat, pl.CRST, p.N, kdim, p.Q, p.P * p.Q,
@@ -54,9 +54,10 @@ static int update_h(const ConvPlan& pl, const void* I, const void* E, void* grad
             // (C * 9 rows of 3x3 filters over 64 k channels divide evenly) and the
             // pixel range is long: a wavefront then multiplies three row blocks with
             // each fragment of E it reads (VGG conv1.2 0.63 -> 0.51 ms, conv2.1
-            // 0.190 -> 0.166 ms)
+            // 0.190 -> 0.166 ms; at 28x28 and 55x55 pixels the 128-row tiles,
+            // which cut the contraction into fewer slices, are 7-10 % faster)
             const bool rows192 = cdiv(pl.CRST, 192) * 192 <= cdiv(pl.CRST, 128) * 128 &&
-                                 (long)pl.p.M * pl.p.P * pl.p.Q * pl.p.N >= 512 * 64;
+                                 (long)pl.p.M * pl.p.P * pl.p.Q * pl.p.N >= 4096 * 64;
             if (pl.p.K <= 64) {
                 if (rows192) return launch_update<_Float16, TIN, TOUT, true, 192, 64, 64, 2, 2>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
                 return launch_update<_Float16, TIN, TOUT, true, 128, 64, 64, 2, 2>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
