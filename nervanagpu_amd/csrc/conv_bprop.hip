@@ -136,30 +136,39 @@ static int bprop_class(const ConvPlan& pl, const BpropClass& c, const void* F, c
     }
 }
 
-// Unit strides, filter rows of three taps, N = 64: the taps of a filter row share
-// one tile of E (see FilterTapColsLoader); a 256-column tile is four pixels of
-// one row of the input image.
+// Unit strides, filter rows of three taps, N = 64 or 128: the taps of a filter row
+// share one tile of E (see FilterTapColsLoader); a 256-column tile is four pixels
+// (N = 64) or two (N = 128) of one row of the input image.
 static bool shares_taps(const ConvPlan& pl)
 {
     const ng_conv_params& p = pl.p;
-    return p.S == 3 && p.N == 64 && p.W % 4 == 0 && p.K % 32 == 0 &&
+    // 128 images: image rows of an odd number of pixels are padded by one if that wastes
+    // at most a twelfth of the columns (the epilogue folds the padding away)
+    const bool rows_fit = p.N == 128 ? 12 * (p.W % 2) <= p.W + p.W % 2 : p.W % 4 == 0;
+    return p.S == 3 && (p.N == 64 || p.N == 128) && rows_fit && p.K % 32 == 0 &&
            p.str_d == 1 && p.str_h == 1 && p.str_w == 1 && !pl.merged;
 }
 
-template <int BM, int WM, int WN, int BN = 256>
+template <int BM, int WM, int WN, int BN = 256, int COLS = 64, int PX = 4>
 static int bprop_shared_taps(const ConvPlan& pl, const void* F, const void* E, void* gradI, float alpha,
                              const void* mask, hipStream_t stream, int col_begin = 0, int col_end = -1)
 {
     typedef _Float16 T;
-    constexpr int BK = 32, TAPS = 3, COLS = 64;
-    static_assert(BN == 4 * COLS || BN == COLS, "four pixels per tile, or one (tail launch)");
+    constexpr int BK = 32, TAPS = 3;
+    static_assert(BN == PX * COLS || BN == COLS, "PX pixels per tile, or one (tail launch)");
     const ng_conv_params& p = pl.p;
-    const int ncols = p.D * p.H * p.W * p.N;
+    const int wpad = cdiv(p.W, PX) * PX;
+    const int ncols = p.D * p.H * wpad * p.N;           // the kernel's columns: padded image rows
+    const int out_cols = p.D * p.H * p.W * p.N;
     const int TR = p.T * p.R, nblk = cdiv(p.K, BK);
-    ScaleStoreEpilogue<T> epi{(T*)gradI, 0, ncols, p.C, ncols, alpha, 0.0f, 0u, 0u, 0u, 0u, 1u, (const T*)mask};
+    ScaleStoreEpilogue<T> epi{(T*)gradI, 0, out_cols, p.C, out_cols, alpha, 0.0f, 0u, 0u, 0u, 0u, 1u, (const T*)mask};
+    if (wpad != p.W) {
+        epi.fold_from = wpad * p.N; epi.fold_to = p.W * p.N;
+        epi.fold_div = FastDiv::make((unsigned)epi.fold_from);
+    }
     FilterTapColsLoader<T, BK, TAPS> al{(const T*)F, p.C, p.K, pl.RST * p.K, FastDiv::make((unsigned)TR),
                                         FastDiv::make((unsigned)p.R), TR, p.R};
-    GatherRowSegLoader<T, BK, TAPS, COLS> bl{(const T*)E, PixelLattice::make(p.N, ncols, p.W, p.H * p.W), p.M, p.P, p.Q,
+    GatherRowSegLoader<T, BK, TAPS, COLS> bl{(const T*)E, PixelLattice::make(p.N, ncols, wpad, p.H * wpad), p.M, p.P, p.Q,
                                              p.T - 1 - p.pad_d, p.R - 1 - p.pad_h, p.S - 1 - p.pad_w,
                                              p.M * p.P * p.Q * p.N,
                                              FastDiv::make((unsigned)TR), FastDiv::make((unsigned)p.R), TR, p.R, p.K};
@@ -257,7 +266,19 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
     }
     if constexpr (sizeof(T) == 2) {
         if (thin_channels(pl, mask)) return bprop_thin(pl, F, E, gradI, alpha, stream);
-        if (shares_taps(pl)) {
+        if (shares_taps(pl) && p.N == 128) {
+            // padded image rows can cost a round over the chip more than the separate taps need
+            double cost, cost_plain;
+            const int row_tile = pick_row_tile(p.C, p.D * p.H * cdiv(p.W, 2) * 2 * p.N, 256, &cost);
+            pick_row_tile(p.C, p.D * p.H * p.W * p.N, 256, &cost_plain);
+            if (cost <= cost_plain) {
+                switch (row_tile) {
+                case 256: return bprop_shared_taps<256, 2, 4, 256, 128, 2>(pl, F, E, gradI, alpha, mask, stream);
+                case 128: return bprop_shared_taps<128, 2, 4, 256, 128, 2>(pl, F, E, gradI, alpha, mask, stream);
+                default:  break;    // 64-row tiles: the separate taps, two workgroups per CU
+                }
+            }
+        } else if (shares_taps(pl)) {
             const int ncols = p.D * p.H * p.W * p.N;
             const int row_tile = pick_row_tile(p.C, ncols, 256);
             // trailing column tiles beyond whole rounds: 64x64 tiles behind the main launch

@@ -31,30 +31,34 @@ static int fprop_tile(const ConvPlan& pl, const void* I, const void* F, void* O,
 }
 
 // Filter rows of three taps on unit strides share their activation tile (see
-// GatherRowSegLoader): N = 64 images, so a 256-column tile is four output pixels
-// of one image row and the shared tile is six input pixels wide.
+// GatherRowSegLoader): a 256-column tile is four output pixels of one image row
+// for N = 64 images (two for N = 128; N = 32 runs 128-column tiles of four), and
+// the shared tile is two input pixels wider.
+static int tap_share_pixels(int N) { return N == 128 ? 2 : 4; }
+
 static bool shares_taps(const ConvPlan& pl)
 {
     const ng_conv_params& p = pl.p;
     // image rows that are not a whole number of tiles are padded to one if that
     // wastes at most a twelfth of the columns (the epilogue folds them away)
-    const int qpad = cdiv(p.Q, 4) * 4;
-    return p.S == 3 && (p.N == 64 || p.N == 32) && 12 * (qpad - p.Q) <= qpad && p.C % 32 == 0 &&
+    const int px = tap_share_pixels(p.N);
+    const int qpad = cdiv(p.Q, px) * px;
+    return p.S == 3 && (p.N == 64 || p.N == 32 || p.N == 128) && 12 * (qpad - p.Q) <= qpad && p.C % 32 == 0 &&
            p.str_d == 1 && p.str_h == 1 && p.str_w == 1;
 }
 
 // COLS = N images per pixel; a tile of BN columns is BN / COLS output pixels of one
-// image row (four, or one for the 64-column tiles of a tail launch); the image rows are
-// padded to a multiple of four pixels
-template <int BM, int WM, int WN, int BN = 256, int COLS = 64>
+// image row (PX of them, or one for the narrow tiles of a tail launch); the image
+// rows are padded to a multiple of PX pixels
+template <int BM, int WM, int WN, int BN = 256, int COLS = 64, int PX = 4>
 static int fprop_shared_taps(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags,
                              hipStream_t stream, int col_begin = 0, int col_end = -1)
 {
     typedef _Float16 T;
     constexpr int BK = 32, TAPS = 3;
-    static_assert(BN == 4 * COLS || BN == COLS, "four output pixels per tile, or one");
+    static_assert(BN == PX * COLS || BN == COLS, "PX output pixels per tile, or one");
     const ng_conv_params& p = pl.p;
-    const int qpad = cdiv(p.Q, 4) * 4;
+    const int qpad = cdiv(p.Q, PX) * PX;
     const int ncols = p.M * p.P * qpad * p.N;           // the kernel's columns: padded image rows
     const int out_cols = p.M * p.P * p.Q * p.N;
     const int TR = p.T * p.R, nblk = cdiv(p.C, BK);
@@ -107,6 +111,21 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
         if (shares_taps(pl) && pl.p.N == 32) {
             // 32 images: 128-column tiles; 128 rows on four wavefronts
             if (pl.p.K >= 128) return fprop_shared_taps<128, 2, 2, 128, 32>(pl, I, F, O, alpha, flags, st);
+        } else if (shares_taps(pl) && pl.p.N == 128) {
+            // 128 images: two output pixels per tile, the shared tile is four wide
+            const int ncols = pl.p.M * pl.p.P * cdiv(pl.p.Q, 2) * 2 * pl.p.N;
+            // padded image rows can push the grid into one more round over the chip
+            // than the unpadded columns of the separate taps need: not worth it then
+            double cost, cost_plain;
+            const int row_tile = pick_row_tile(pl.p.K, ncols, 256, &cost);
+            pick_row_tile(pl.p.K, pl.p.M * pl.p.P * pl.p.Q * pl.p.N, 256, &cost_plain);
+            if (cost <= cost_plain) {
+                switch (row_tile) {
+                case 256: return fprop_shared_taps<256, 2, 4, 256, 128, 2>(pl, I, F, O, alpha, flags, st);
+                case 128: return fprop_shared_taps<128, 2, 4, 256, 128, 2>(pl, I, F, O, alpha, flags, st);
+                default:  break;    // 64-row tiles: the separate taps, two workgroups per CU
+                }
+            }
         } else if (shares_taps(pl)) {
             const int ncols = pl.p.M * pl.p.P * cdiv(pl.p.Q, 4) * 4 * pl.p.N;
             const int row_tile = pick_row_tile(pl.p.K, ncols, 256);

@@ -100,7 +100,7 @@ inline int check_ptr16(const void* p, const char* what)
 // 64-row problem with many column tiles picks the 64-row tile, while a grid of
 // at most one workgroup per CU prefers the 128-row tile, whose eight wavefronts
 // hide the latency of a tile step better.
-inline int pick_row_tile(int rows, int ncols, int bn)
+inline int pick_row_tile(int rows, int ncols, int bn, double* cost_out = nullptr)
 {
     static const int tiles[3] = {256, 128, 64};
     static const int resident[3] = {1, 1, 2};
@@ -114,6 +114,7 @@ inline int pick_row_tile(int rows, int ncols, int bn)
         const double cost = (double)((blocks + slots - 1) / slots) * step_us[i];
         if (i == 0 || cost < best_cost * 0.999) { best = tiles[i]; best_cost = cost; }
     }
+    if (cost_out) *cost_out = best_cost;
     return best;
 }
 

@@ -45,8 +45,13 @@ static int update_h(const ConvPlan& pl, const void* I, const void* E, void* grad
         // fp16 activations: tile shaped after the filter matrix (CRST x K)
         if constexpr (std::is_same<TIN, _Float16>::value) {
             // 256x256 tiles leave few output tiles, i.e. many contraction slices
-            // and fp32 partials: worth it only for long pixel ranges
-            if (pl.p.K >= 256 && pl.CRST >= 256 && (long)pl.p.M * pl.p.P * pl.p.Q * pl.p.N >= 512 * 64)
+            // and fp32 partials: worth it for long pixel ranges, or when the filter
+            // is so large that the 128x128 tiles take more than one round of the
+            // chip without any slicing (512 -> 1024 maps on 12x12 pixels, N = 128:
+            // 0.259 -> 0.200 ms)
+            const long kdim = (long)pl.p.M * pl.p.P * pl.p.Q * pl.p.N;
+            const long tiles128 = (long)cdiv(pl.CRST, 128) * cdiv(pl.p.K, 128);
+            if (pl.p.K >= 256 && pl.CRST >= 256 && (kdim >= 512 * 64 || tiles128 > device_cu_count()))
                 return launch_update<_Float16, TIN, TOUT, true, 256, 256, 64, 2, 4>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
             if (pl.p.K <= 64 && pl.CRST <= 64)
                 return launch_update<_Float16, TIN, TOUT, true, 64, 64, 64, 2, 2>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
@@ -56,8 +61,7 @@ static int update_h(const ConvPlan& pl, const void* I, const void* E, void* grad
             // each fragment of E it reads (VGG conv1.2 0.63 -> 0.51 ms, conv2.1
             // 0.190 -> 0.166 ms; at 28x28 and 55x55 pixels the 128-row tiles,
             // which cut the contraction into fewer slices, are 7-10 % faster)
-            const bool rows192 = cdiv(pl.CRST, 192) * 192 <= cdiv(pl.CRST, 128) * 128 &&
-                                 (long)pl.p.M * pl.p.P * pl.p.Q * pl.p.N >= 4096 * 64;
+            const bool rows192 = cdiv(pl.CRST, 192) * 192 <= cdiv(pl.CRST, 128) * 128 && kdim >= 4096 * 64;
             if (pl.p.K <= 64) {
                 if (rows192) return launch_update<_Float16, TIN, TOUT, true, 192, 64, 64, 2, 2>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
                 return launch_update<_Float16, TIN, TOUT, true, 128, 64, 64, 2, 2>(pl, I, E, gradF, alpha, ws, ws_bytes, st);

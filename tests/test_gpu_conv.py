@@ -66,6 +66,14 @@ SMALL = [
     # second launch (forward with 128 output maps; data gradient with 128 channels)
     (64, 32, 128, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     (64, 128, 32, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    # 128 images: shared taps with two pixels per 256-column tile (128- and 256-row tiles, forward with
+    # 13-pixel output rows padded to 14 and folded, 3-D without horizontal padding, data gradient of 512 channels)
+    (128, 32, 128, 1, 6, 8, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (128, 32, 128, 1, 5, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (128, 64, 160, 2, 5, 8, 2, 3, 3, (1, 0, 0), (1, 1, 1)),
+    (128, 32, 512, 1, 10, 14, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (128, 512, 32, 1, 10, 14, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (128, 64, 32, 1, 4, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1)),          # data gradient with 13-pixel image rows padded to 14
     # long pixel ranges with filter rows in multiples of 192: the weight gradient's 192-row tiles
     (64, 64, 32, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     (64, 64, 96, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
@@ -75,7 +83,10 @@ SMALL = [
 # cases that exist for a half-precision kernel and are large
 FP16_ONLY = {(64, 3, 64, 1, 20, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 5, 32, 1, 24, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
              (32, 32, 128, 2, 5, 8, 2, 3, 3, (1, 1, 1), (1, 1, 1)), (32, 64, 136, 1, 6, 12, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
-             (64, 32, 128, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 128, 32, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1))}
+             (64, 32, 128, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 128, 32, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+             (128, 32, 512, 1, 10, 14, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (128, 512, 32, 1, 10, 14, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+             (128, 64, 160, 2, 5, 8, 2, 3, 3, (1, 0, 0), (1, 1, 1)), (128, 32, 128, 1, 6, 8, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+             (128, 32, 128, 1, 5, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (128, 64, 32, 1, 4, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1))}
 
 
 def _layer(ng, dtype, case):
@@ -352,7 +363,9 @@ def test_bprop_with_rectifier_mask(ng, dtype):
                  (64, 72, 96, 1, 5, 12, 1, 3, 3, (0, 0, 0), (1, 1, 1)),        # shared taps
                  (64, 32, 64, 3, 4, 8, 3, 2, 3, (2, 0, 1), (1, 1, 1)),         # shared taps, 3-D
                  (16, 64, 64, 1, 20, 20, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
-                 (64, 128, 32, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1))):     # main launch + tail launch
+                 (64, 128, 32, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)),      # main launch + tail launch
+                 (128, 32, 128, 1, 6, 8, 1, 3, 3, (0, 1, 1), (1, 1, 1)),       # shared taps, 128 images
+                 (128, 64, 32, 1, 4, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1))):      # ... with padded image rows
         if dtype == np.float32 and case in FP16_ONLY:
             continue
         layer = _layer(ng, dtype, case)
