@@ -106,7 +106,7 @@ static int run_bprop_merged(const ConvPlan& pl, const void* F, const void* E, vo
 
 template <typename T, bool BLOCKED, int BM, int BN, int BK, int WM, int WN>
 static int bprop_class(const ConvPlan& pl, const BpropClass& c, const void* F, const T* Fs, const void* E, void* gradI,
-                       float alpha, const void* mask, hipStream_t stream)
+                       float alpha, const void* mask, hipStream_t stream, int col_begin = 0, int col_end = -1)
 {
     const ng_conv_params& p = pl.p;
     const int ncols = c.nz * c.ny * c.nx * p.N;
@@ -127,12 +127,12 @@ static int bprop_class(const ConvPlan& pl, const BpropClass& c, const void* F, c
         // the filter is read in place: rows c, contraction (tap, k)
         FilterRowsLoader<T, BK> al{(const T*)F, pl.d_bprop_trs + c.tap_offset, p.C, p.K, pl.RST * p.K,
                                    FastDiv::make((unsigned)std::max(c.taps, 1)), c.taps};
-        if (dense) return launch_core<T, BM, BN, BK, WM, WN, KC, MC>(al, bl, depi, p.C, ncols, k_tiles, 1, stream, "conv bprop");
-        return launch_core<T, BM, BN, BK, WM, WN, KC, MC>(al, bl, lepi, p.C, ncols, k_tiles, 1, stream, "conv bprop");
+        if (dense) return launch_core<T, BM, BN, BK, WM, WN, KC, MC>(al, bl, depi, p.C, ncols, k_tiles, 1, stream, "conv bprop", col_begin, col_end);
+        return launch_core<T, BM, BN, BK, WM, WN, KC, MC>(al, bl, lepi, p.C, ncols, k_tiles, 1, stream, "conv bprop", col_begin, col_end);
     } else {
         DenseLoader<T, MC, true> al{Fs + c.w_row * pl.Cpad, 0, pl.Cpad, pl.Cpad, c.J};
-        if (dense) return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, depi, p.C, ncols, k_tiles, 1, stream, "conv bprop");
-        return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, lepi, p.C, ncols, k_tiles, 1, stream, "conv bprop");
+        if (dense) return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, depi, p.C, ncols, k_tiles, 1, stream, "conv bprop", col_begin, col_end);
+        return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, lepi, p.C, ncols, k_tiles, 1, stream, "conv bprop", col_begin, col_end);
     }
 }
 
@@ -235,7 +235,19 @@ template <bool BLOCKED>
 static int bprop_class_h(const ConvPlan& pl, const BpropClass& c, const void* F, const _Float16* Fs, const void* E,
                          void* gradI, float alpha, const void* mask, hipStream_t st)
 {
-    switch (pick_row_tile(pl.p.C, c.nz * c.ny * c.nx * pl.p.N, 256)) {
+    const int ncols = c.nz * c.ny * c.nx * pl.p.N;
+    const int row_tile = pick_row_tile(pl.p.C, ncols, 256);
+    if constexpr (BLOCKED) {
+        // trailing column tiles beyond whole rounds: 64x64 tiles behind the main launch
+        const int tail = row_tile >= 128 ? tail_column_tiles(cdiv(pl.p.C, row_tile), cdiv(ncols, 256)) : 0;
+        if (tail) {
+            const int cut = (cdiv(ncols, 256) - tail) * 256;
+            const int rc = row_tile == 256 ? bprop_class<_Float16, BLOCKED, 256, 256, 64, 2, 4>(pl, c, F, Fs, E, gradI, alpha, mask, st, 0, cut)
+                                           : bprop_class<_Float16, BLOCKED, 128, 256, 64, 2, 4>(pl, c, F, Fs, E, gradI, alpha, mask, st, 0, cut);
+            return rc ? rc : bprop_class<_Float16, BLOCKED, 64, 64, 64, 2, 2>(pl, c, F, Fs, E, gradI, alpha, mask, st, cut, -1);
+        }
+    }
+    switch (row_tile) {
     case 256: return bprop_class<_Float16, BLOCKED, 256, 256, 64, 2, 4>(pl, c, F, Fs, E, gradI, alpha, mask, st);
     case 128: return bprop_class<_Float16, BLOCKED, 128, 256, 64, 2, 4>(pl, c, F, Fs, E, gradI, alpha, mask, st);
     default:  return bprop_class<_Float16, BLOCKED, 64, 256, 64, 1, 4>(pl, c, F, Fs, E, gradI, alpha, mask, st);

@@ -6,7 +6,7 @@ namespace ng {
 
 template <typename T, typename TIN, bool BLOCKED, int BM, int BN, int BK, int WM, int WN, int NSTAGE = 2>
 static int fprop_tile(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags,
-                      hipStream_t stream)
+                      hipStream_t stream, int col_begin = 0, int col_end = -1)
 {
     const ng_conv_params& p = pl.p;
     const int ncols = p.M * p.P * p.Q * p.N;
@@ -20,13 +20,15 @@ static int fprop_tile(const ConvPlan& pl, const void* I, const void* F, void* O,
         GatherColsLoader<T, TIN, true, BK> bl{(const TIN*)I, pl.d_fprop_taps, pl.CRST, lat,
                                               p.str_d, p.str_h, p.str_w, p.D, p.H, p.W,
                                               DHWN, FastDiv::make((unsigned)pl.RST), nblk, p.C, pl.RST, pl.RST};
-        return launch_core<T, BM, BN, BK, WM, WN, MC, MC, NSTAGE>(al, bl, epi, p.K, ncols, pl.RST * nblk, 1, stream, "conv fprop");
+        return launch_core<T, BM, BN, BK, WM, WN, MC, MC, NSTAGE>(al, bl, epi, p.K, ncols, pl.RST * nblk, 1, stream, "conv fprop",
+                                                                  col_begin, col_end);
     } else {
         DenseLoader<T, MC, true> al{(const T*)F, 0, p.K, p.K, pl.CRST};
         GatherColsLoader<T, TIN, false, BK> bl{(const TIN*)I, pl.d_fprop_flat, pl.CRST, lat,
                                                p.str_d, p.str_h, p.str_w, p.D, p.H, p.W,
                                                0, FastDiv{0, 0}, 1, 0, 0};
-        return launch_core<T, BM, BN, BK, WM, WN, MC, MC, NSTAGE>(al, bl, epi, p.K, ncols, cdiv(pl.CRST, BK), 1, stream, "conv fprop");
+        return launch_core<T, BM, BN, BK, WM, WN, MC, MC, NSTAGE>(al, bl, epi, p.K, ncols, cdiv(pl.CRST, BK), 1, stream, "conv fprop",
+                                                                  col_begin, col_end);
     }
 }
 
@@ -155,7 +157,20 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
             }
         }
     }
-    switch (pick_row_tile(pl.p.K, pl.p.M * pl.p.P * pl.p.Q * pl.p.N, 256)) {
+    const int ncols = pl.p.M * pl.p.P * pl.p.Q * pl.p.N;
+    const int row_tile = pick_row_tile(pl.p.K, ncols, 256);
+    if constexpr (BLOCKED && std::is_same<TIN, _Float16>::value) {
+        // as with the shared taps: the few column tiles beyond whole rounds of one-per-CU
+        // workgroups run behind the main launch as 64x64 tiles
+        const int tail = row_tile >= 128 ? tail_column_tiles(cdiv(pl.p.K, row_tile), cdiv(ncols, 256)) : 0;
+        if (tail) {
+            const int cut = (cdiv(ncols, 256) - tail) * 256;
+            const int rc = row_tile == 256 ? fprop_tile<_Float16, TIN, BLOCKED, 256, 256, 64, 2, 4>(pl, I, F, O, alpha, flags, st, 0, cut)
+                                           : fprop_tile<_Float16, TIN, BLOCKED, 128, 256, 64, 2, 4>(pl, I, F, O, alpha, flags, st, 0, cut);
+            return rc ? rc : fprop_tile<_Float16, TIN, BLOCKED, 64, 64, 64, 2, 2>(pl, I, F, O, alpha, flags, st, cut, -1);
+        }
+    }
+    switch (row_tile) {
     case 256: return fprop_tile<_Float16, TIN, BLOCKED, 256, 256, 64, 2, 4>(pl, I, F, O, alpha, flags, st);
     // 128 rows on eight wavefronts: mid-sized layers run about one workgroup per
     // CU, and twice the wavefronts hide the LDS and request latency of a tile

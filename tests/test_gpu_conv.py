@@ -74,6 +74,10 @@ SMALL = [
     (128, 32, 512, 1, 10, 14, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     (128, 512, 32, 1, 10, 14, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     (128, 64, 32, 1, 4, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1)),          # data gradient with 13-pixel image rows padded to 14
+    # the same tail launch on the kernels with separate taps (16 images: forward with 128 output maps,
+    # data gradient with 128 channels, 288 column tiles each)
+    (16, 64, 128, 1, 64, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (16, 128, 64, 1, 64, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     # long pixel ranges with filter rows in multiples of 192: the weight gradient's 192-row tiles
     (64, 64, 32, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     (64, 64, 96, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
@@ -86,7 +90,8 @@ FP16_ONLY = {(64, 3, 64, 1, 20, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 5, 32, 
              (64, 32, 128, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 128, 32, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
              (128, 32, 512, 1, 10, 14, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (128, 512, 32, 1, 10, 14, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
              (128, 64, 160, 2, 5, 8, 2, 3, 3, (1, 0, 0), (1, 1, 1)), (128, 32, 128, 1, 6, 8, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
-             (128, 32, 128, 1, 5, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (128, 64, 32, 1, 4, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1))}
+             (128, 32, 128, 1, 5, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (128, 64, 32, 1, 4, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+             (16, 64, 128, 1, 64, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (16, 128, 64, 1, 64, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1))}
 
 
 def _layer(ng, dtype, case):
@@ -365,7 +370,8 @@ def test_bprop_with_rectifier_mask(ng, dtype):
                  (16, 64, 64, 1, 20, 20, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
                  (64, 128, 32, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)),      # main launch + tail launch
                  (128, 32, 128, 1, 6, 8, 1, 3, 3, (0, 1, 1), (1, 1, 1)),       # shared taps, 128 images
-                 (128, 64, 32, 1, 4, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1))):      # ... with padded image rows
+                 (128, 64, 32, 1, 4, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1)),       # ... with padded image rows
+                 (16, 128, 64, 1, 64, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1))):      # separate taps, main + tail launch
         if dtype == np.float32 and case in FP16_ONLY:
             continue
         layer = _layer(ng, dtype, case)
