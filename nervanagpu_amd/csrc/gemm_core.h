@@ -384,8 +384,15 @@ __device__ __forceinline__ void wave_lds_fence()
 template <class E, class = void> struct EpilogueBufferStore { static constexpr bool value = false; };
 template <class E> struct EpilogueBufferStore<E, std::enable_if_t<E::BUFFER_STORE>> { static constexpr bool value = true; };
 
-template <int TM, int TN, int WTN, int EPITCH, int I>
+// ROW_TAPS > 1: the TM bands of a wavefront are ROW_TAPS interleaved row sets (band
+// I holds rows (mbase + (I / ROW_TAPS) * 32 + r) * ROW_TAPS + I % ROW_TAPS: the
+// horizontal taps of 32 filter rows of the weight gradient's ring kernel)
+template <int TM, int TN, int WTN, int EPITCH, int I, int ROW_TAPS = 1>
 struct EpilogueBands {
+    static __device__ __forceinline__ int row_of(int mbase, int r)
+    {
+        return ROW_TAPS == 1 ? mbase + I * 32 + r : (mbase + (I / ROW_TAPS) * 32 + r) * ROW_TAPS + I % ROW_TAPS;
+    }
     template <class Epi>
     static __device__ __forceinline__ void run(float16_t (&acc)[TM][TN], char* stage, int lane,
                                                int mbase, int nbase, int z, int split, const Epi& epi)
@@ -417,7 +424,7 @@ struct EpilogueBands {
                     const float4_t lo = *reinterpret_cast<const float4_t*>(stage + r * EPITCH + cc * 4);
                     const float4_t hi = *reinterpret_cast<const float4_t*>(stage + r * EPITCH + cc * 4 + 16);
                     const float vals[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    epi.store8_buffer(rsrc, mbase + I * 32 + r, nbase + cc, vals);
+                    epi.store8_buffer(rsrc, row_of(mbase, r), nbase + cc, vals);
                 }
             }
         } else {
@@ -429,12 +436,12 @@ struct EpilogueBands {
                 const float4_t lo = *reinterpret_cast<const float4_t*>(stage + r * EPITCH + cc * 4);
                 const float4_t hi = *reinterpret_cast<const float4_t*>(stage + r * EPITCH + cc * 4 + 16);
                 const float vals[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                epi.store8(mbase + I * 32 + r, nbase + cc, z, split, vals);
+                epi.store8(row_of(mbase, r), nbase + cc, z, split, vals);
             }
         }
         wave_lds_fence();
         if constexpr (I + 1 < TM)
-            EpilogueBands<TM, TN, WTN, EPITCH, I + 1>::run(acc, stage, lane, mbase, nbase, z, split, epi);
+            EpilogueBands<TM, TN, WTN, EPITCH, I + 1, ROW_TAPS>::run(acc, stage, lane, mbase, nbase, z, split, epi);
     }
 };
 
