@@ -148,10 +148,11 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
         for (const auto& t : shapes)
             splits = std::max(splits, conv_splits(cdiv(pl->CRST, t[0]) * cdiv(p.K, t[1]), kt, 0, 0, update_tiles_per_cu(t[0], t[1])));
         // the ring kernel of filters with three horizontal taps: 64 or 192 rows (c,t,r) per tile, W + 2 positions per image row
-        if (p.S == 3 && p.K <= 64) {
+        if (p.S == 3 && p.K <= 128) {
             const int ring_steps = p.M * p.P * (p.W + 2), CR = p.C * p.T * p.R;
             splits = std::max(splits, conv_splits(cdiv(CR, 64), ring_steps, 0, 0, 3));
             splits = std::max(splits, conv_splits(cdiv(CR, 192), ring_steps, 0, 0, 1));
+            splits = std::max(splits, conv_splits(cdiv(CR, 128), ring_steps, 0, 0, 1));
         }
         pl->ws_update = splits > 1 ? align_up((size_t)splits * pl->CRST * p.K * sizeof(float), 256) : 0;
     }

@@ -40,12 +40,16 @@ static int launch_update(const ConvPlan& pl, const void* I, const void* E, void*
 
 // Three horizontal taps, unit strides, 64 images, at most 64 output maps and at least 64
 // rows (c,t,r): the ring kernel (conv_update_ring.h).  With more output maps the tiles of
-// gemm_core.h are not bound by their requests and stay faster (64 -> 128 maps on 112x112:
-// 0.143 against 0.160 ms).
+// gemm_core.h are less bound by their requests (64 -> 128 maps on 112x112: 0.143 against
+// 0.160 ms with 64-row workgroups).
 static bool update_shares_taps(const ConvPlan& pl)
 {
     const ng_conv_params& p = pl.p;
-    return p.S == 3 && p.pad_w == 1 && p.N == 64 && p.K <= 64 && p.C * p.T * p.R >= 64 && p.K % 8 == 0 &&
+    const int CR = p.C * p.T * p.R;
+    // 65 .. 128 output maps: only with whole 128-row workgroups on large maps (3-6 % faster than the
+    // general tiles on 96x96 and 112x112 maps; on 56x56 and with padded rows it is a draw or worse)
+    const bool fits = p.K <= 64 ? CR >= 64 : (p.K <= 128 && CR % 128 == 0 && (long)p.M * p.P * p.Q >= 8192);
+    return p.S == 3 && p.pad_w == 1 && p.N == 64 && fits && p.K % 8 == 0 &&
            p.str_d == 1 && p.str_h == 1 && p.str_w == 1 &&
            (long)p.C * p.D * p.H * p.W * p.N * 2 < (1L << 31) && (long)p.K * p.M * p.P * p.Q * p.N * 2 < (1L << 31);
 }
@@ -98,6 +102,7 @@ static int update_h(const ConvPlan& pl, const void* I, const void* E, void* grad
                 // then requested once instead of once per 64 rows; VGG conv1.2 0.47 -> 0.38 ms),
                 // when 192-row tiles pad the rows no more than 64-row tiles do
                 const int CR = pl.p.C * pl.p.T * pl.p.R;
+                if (pl.p.K > 64) return launch_update_ring<TOUT, 128, 128, 1, 1>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
                 if (cdiv(CR, 192) * 192 <= cdiv(CR, 64) * 64)
                     return launch_update_ring<TOUT, 192, 64, 2, 1>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
                 return launch_update_ring<TOUT, 64, 64, 1, 3>(pl, I, E, gradF, alpha, ws, ws_bytes, st);

@@ -1,5 +1,5 @@
 // Weight gradient of filters with three horizontal taps, unit strides and few output
-// maps (at most 64): the taps share their activations.
+// maps (at most 128): the taps share their activations.
 //
 // gF[(c,t,r,s)][k] = sum over output pixels (m,p,q) and images n of
 //                    I[c, m+t-pad_d, p+r-pad_h, q+s-1, n] * E[k, m, p, q, n].

@@ -83,6 +83,8 @@ SMALL = [
     # positions that cross image rows; the other cases with 64 images, 3x3 filters and K <= 64 take it too)
     (64, 120, 24, 1, 5, 9, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     (64, 64, 64, 1, 20, 20, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    # ... and with 65 to 128 output maps on maps of 8192 pixels or more: 128-row workgroups, two column blocks per wavefront
+    (64, 128, 72, 1, 91, 91, 1, 1, 3, (0, 0, 1), (1, 1, 1)),
     # long pixel ranges with filter rows in multiples of 192: the weight gradient's 192-row tiles
     (64, 64, 32, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     (64, 64, 96, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
@@ -97,7 +99,8 @@ FP16_ONLY = {(64, 3, 64, 1, 20, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 5, 32, 
              (128, 64, 160, 2, 5, 8, 2, 3, 3, (1, 0, 0), (1, 1, 1)), (128, 32, 128, 1, 6, 8, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
              (128, 32, 128, 1, 5, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (128, 64, 32, 1, 4, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
              (16, 64, 128, 1, 64, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (16, 128, 64, 1, 64, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
-             (64, 120, 24, 1, 5, 9, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 64, 64, 1, 20, 20, 1, 3, 3, (0, 1, 1), (1, 1, 1))}
+             (64, 120, 24, 1, 5, 9, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 64, 64, 1, 20, 20, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+             (64, 128, 72, 1, 91, 91, 1, 1, 3, (0, 0, 1), (1, 1, 1))}
 
 
 def _layer(ng, dtype, case):
