@@ -82,7 +82,8 @@ void conv_update_ring_kernel(UpdateRingGeom g, Epi epi, CoreShape s)
         int r, k;
         TA::chunk_pos(tid + i * NT, r, k);
         const int cr = cr0 + r;
-        const int c = (int)g.tr_div.div((unsigned)cr), tr = cr - c * g.TR;
+        const int crc = min(cr, g.CR - 1);          // rows past the filter decode as the last row (never read)
+        const int c = (int)g.tr_div.div((unsigned)crc), tr = crc - c * g.TR;
         const int t = (int)g.r_div.div((unsigned)tr), rf = tr - t * g.R;
         a_dz[i] = (cr < g.CR) ? t - g.pad_d : (1 << 20);       // rows past the filter never pass the range test
         a_dy[i] = rf - g.pad_h;
