@@ -166,8 +166,10 @@ int ng_conv_plan_create(const ng_conv_params* p, int dtype, void** plan);
 int ng_conv_plan_destroy(void* plan);
 /* scratch bytes the three conv ops may use for this plan (filter re-layout for
  * the bprop of layers with few channels or output maps, split partial sums for
- * update; may be 0); the reference keeps one shared scratch buffer for the
- * same two purposes (nervanagpu/nervanagpu.py:686-698) */
+ * update and for fprop / bprop grids much smaller than the chip; may be 0); the
+ * reference keeps one shared scratch buffer for the first two purposes
+ * (nervanagpu/nervanagpu.py:686-698).  fprop, and bprop when it needs no filter
+ * re-layout, also run without a workspace (unsliced). */
 size_t ng_conv_plan_workspace_bytes(const void* plan);
 /* O = round(relu?(alpha * conv(I, F))).  in_dtype may be NG_U8/NG_I8 with
  * NG_F16 filters and output: the bytes are converted exactly on load (declared

@@ -106,7 +106,8 @@ static int run_bprop_merged(const ConvPlan& pl, const void* F, const void* E, vo
 
 template <typename T, bool BLOCKED, int BM, int BN, int BK, int WM, int WN>
 static int bprop_class(const ConvPlan& pl, const BpropClass& c, const void* F, const T* Fs, const void* E, void* gradI,
-                       float alpha, const void* mask, hipStream_t stream, int col_begin = 0, int col_end = -1)
+                       float alpha, const void* mask, hipStream_t stream, int col_begin = 0, int col_end = -1,
+                       void* ws = nullptr, size_t ws_bytes = 0)
 {
     const ng_conv_params& p = pl.p;
     const int ncols = c.nz * c.ny * c.nx * p.N;
@@ -127,6 +128,9 @@ static int bprop_class(const ConvPlan& pl, const BpropClass& c, const void* F, c
         // the filter is read in place: rows c, contraction (tap, k)
         FilterRowsLoader<T, BK> al{(const T*)F, pl.d_bprop_trs + c.tap_offset, p.C, p.K, pl.RST * p.K,
                                    FastDiv::make((unsigned)std::max(c.taps, 1)), c.taps};
+        // the filter is read in place, so the scratch is free for contraction slices of a small grid
+        if (dense && col_begin == 0 && col_end < 0)
+            return launch_core_sliced<T, BM, BN, BK, WM, WN, KC, MC>(al, bl, depi, p.C, ncols, k_tiles, ws, ws_bytes, stream, "conv bprop");
         if (dense) return launch_core<T, BM, BN, BK, WM, WN, KC, MC>(al, bl, depi, p.C, ncols, k_tiles, 1, stream, "conv bprop", col_begin, col_end);
         return launch_core<T, BM, BN, BK, WM, WN, KC, MC>(al, bl, lepi, p.C, ncols, k_tiles, 1, stream, "conv bprop", col_begin, col_end);
     } else {
@@ -233,7 +237,7 @@ static int bprop_thin(const ConvPlan& pl, const void* F, const void* E, void* gr
 
 template <bool BLOCKED>
 static int bprop_class_h(const ConvPlan& pl, const BpropClass& c, const void* F, const _Float16* Fs, const void* E,
-                         void* gradI, float alpha, const void* mask, hipStream_t st)
+                         void* gradI, float alpha, const void* mask, hipStream_t st, void* ws, size_t ws_bytes)
 {
     const int ncols = c.nz * c.ny * c.nx * pl.p.N;
     const int row_tile = pick_row_tile(pl.p.C, ncols, 256);
@@ -248,9 +252,9 @@ static int bprop_class_h(const ConvPlan& pl, const BpropClass& c, const void* F,
         }
     }
     switch (row_tile) {
-    case 256: return bprop_class<_Float16, BLOCKED, 256, 256, 64, 2, 4>(pl, c, F, Fs, E, gradI, alpha, mask, st);
-    case 128: return bprop_class<_Float16, BLOCKED, 128, 256, 64, 2, 4>(pl, c, F, Fs, E, gradI, alpha, mask, st);
-    default:  return bprop_class<_Float16, BLOCKED, 64, 256, 64, 1, 4>(pl, c, F, Fs, E, gradI, alpha, mask, st);
+    case 256: return bprop_class<_Float16, BLOCKED, 256, 256, 64, 2, 4>(pl, c, F, Fs, E, gradI, alpha, mask, st, 0, -1, ws, ws_bytes);
+    case 128: return bprop_class<_Float16, BLOCKED, 128, 256, 64, 2, 4>(pl, c, F, Fs, E, gradI, alpha, mask, st, 0, -1, ws, ws_bytes);
+    default:  return bprop_class<_Float16, BLOCKED, 64, 256, 64, 1, 4>(pl, c, F, Fs, E, gradI, alpha, mask, st, 0, -1, ws, ws_bytes);
     }
 }
 
@@ -262,6 +266,8 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
     // the mask shares the plain store epilogue's indexing: unit strides only
     if (mask && (pl.merged || p.str_d != 1 || p.str_h != 1 || p.str_w != 1))
         return fail(-51, "ng_conv_bprop: the rectifier mask needs unit strides");
+    // no scratch is required when the filter is read in place; an aligned one may hold contraction slices
+    if (!pl.ws_bprop && ((uintptr_t)ws & 15)) { ws = nullptr; ws_bytes = 0; }
     if (pl.ws_bprop && (ws_bytes < pl.ws_bprop || !ws))
         return fail(-40, "ng_conv_bprop: workspace too small (%zu < %zu)", ws_bytes, pl.ws_bprop);
     if (pl.merged)
@@ -312,10 +318,10 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
         if (c.nz * c.ny * c.nx == 0) continue;
         int rc;
         if (sizeof(T) == 2)
-            rc = blocked ? bprop_class_h<true>(pl, c, F, (const _Float16*)Fs, E, gradI, alpha, mask, stream)
-                         : bprop_class_h<false>(pl, c, F, (const _Float16*)Fs, E, gradI, alpha, mask, stream);
+            rc = blocked ? bprop_class_h<true>(pl, c, F, (const _Float16*)Fs, E, gradI, alpha, mask, stream, ws, ws_bytes)
+                         : bprop_class_h<false>(pl, c, F, (const _Float16*)Fs, E, gradI, alpha, mask, stream, nullptr, 0);
         else
-            rc = blocked ? bprop_class<float, true, 128, 128, 16, 2, 2>(pl, c, F, (const float*)Fs, E, gradI, alpha, mask, stream)
+            rc = blocked ? bprop_class<float, true, 128, 128, 16, 2, 2>(pl, c, F, (const float*)Fs, E, gradI, alpha, mask, stream, 0, -1, ws, ws_bytes)
                          : bprop_class<float, false, 128, 128, 16, 2, 2>(pl, c, F, (const float*)Fs, E, gradI, alpha, mask, stream);
         if (rc) return rc;
     }

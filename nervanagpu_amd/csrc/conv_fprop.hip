@@ -6,8 +6,9 @@ namespace ng {
 
 template <typename T, typename TIN, bool BLOCKED, int BM, int BN, int BK, int WM, int WN, int NSTAGE = 2>
 static int fprop_tile(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags,
-                      hipStream_t stream, int col_begin = 0, int col_end = -1)
+                      hipStream_t stream, int col_begin = 0, int col_end = -1, void* ws = nullptr, size_t ws_bytes = 0)
 {
+    const bool whole = col_begin == 0 && col_end < 0;     // a launch over all columns may slice its contraction
     const ng_conv_params& p = pl.p;
     const int ncols = p.M * p.P * p.Q * p.N;
     const int DHWN = p.D * p.H * p.W * p.N;
@@ -20,6 +21,7 @@ static int fprop_tile(const ConvPlan& pl, const void* I, const void* F, void* O,
         GatherColsLoader<T, TIN, true, BK> bl{(const TIN*)I, pl.d_fprop_taps, pl.CRST, lat,
                                               p.str_d, p.str_h, p.str_w, p.D, p.H, p.W,
                                               DHWN, FastDiv::make((unsigned)pl.RST), nblk, p.C, pl.RST, pl.RST};
+        if (whole) return launch_core_sliced<T, BM, BN, BK, WM, WN, MC, MC, NSTAGE>(al, bl, epi, p.K, ncols, pl.RST * nblk, ws, ws_bytes, stream, "conv fprop");
         return launch_core<T, BM, BN, BK, WM, WN, MC, MC, NSTAGE>(al, bl, epi, p.K, ncols, pl.RST * nblk, 1, stream, "conv fprop",
                                                                   col_begin, col_end);
     } else {
@@ -27,6 +29,7 @@ static int fprop_tile(const ConvPlan& pl, const void* I, const void* F, void* O,
         GatherColsLoader<T, TIN, false, BK> bl{(const TIN*)I, pl.d_fprop_flat, pl.CRST, lat,
                                                p.str_d, p.str_h, p.str_w, p.D, p.H, p.W,
                                                0, FastDiv{0, 0}, 1, 0, 0};
+        if (whole) return launch_core_sliced<T, BM, BN, BK, WM, WN, MC, MC, NSTAGE>(al, bl, epi, p.K, ncols, cdiv(pl.CRST, BK), ws, ws_bytes, stream, "conv fprop");
         return launch_core<T, BM, BN, BK, WM, WN, MC, MC, NSTAGE>(al, bl, epi, p.K, ncols, cdiv(pl.CRST, BK), 1, stream, "conv fprop",
                                                                   col_begin, col_end);
     }
@@ -107,7 +110,8 @@ static bool streams_columns(const ConvPlan& pl)
 }
 
 template <typename TIN, bool BLOCKED>
-static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags, hipStream_t st)
+static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags, hipStream_t st,
+                   void* ws, size_t ws_bytes)
 {
     if constexpr (BLOCKED && std::is_same<TIN, _Float16>::value) {
         if (shares_taps(pl) && pl.p.N == 32) {
@@ -171,16 +175,16 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
         }
     }
     switch (row_tile) {
-    case 256: return fprop_tile<_Float16, TIN, BLOCKED, 256, 256, 64, 2, 4>(pl, I, F, O, alpha, flags, st);
+    case 256: return fprop_tile<_Float16, TIN, BLOCKED, 256, 256, 64, 2, 4>(pl, I, F, O, alpha, flags, st, 0, -1, ws, ws_bytes);
     // 128 rows on eight wavefronts: mid-sized layers run about one workgroup per
     // CU, and twice the wavefronts hide the LDS and request latency of a tile
-    case 128: return fprop_tile<_Float16, TIN, BLOCKED, 128, 256, 64, 2, 4>(pl, I, F, O, alpha, flags, st);
+    case 128: return fprop_tile<_Float16, TIN, BLOCKED, 128, 256, 64, 2, 4>(pl, I, F, O, alpha, flags, st, 0, -1, ws, ws_bytes);
     default:
         // Row-by-row gathered contractions (first layers, few channels) are bound
         // by request latency, not by the matrix pipe: half-depth tiles halve the
         // LDS footprint, so twice as many workgroups per CU keep requests in flight
-        if (!BLOCKED) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 32, 1, 4>(pl, I, F, O, alpha, flags, st);
-        return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 64, 1, 4>(pl, I, F, O, alpha, flags, st);
+        if (!BLOCKED) return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 32, 1, 4>(pl, I, F, O, alpha, flags, st, 0, -1, ws, ws_bytes);
+        return fprop_tile<_Float16, TIN, BLOCKED, 64, 256, 64, 1, 4>(pl, I, F, O, alpha, flags, st, 0, -1, ws, ws_bytes);
     }
 }
 
@@ -189,7 +193,7 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
 using namespace ng;
 
 extern "C" int ng_conv_fprop(const void* plan, int in_dtype, const void* I, const void* F, void* O,
-                             float alpha, unsigned flags, void* /*workspace*/, size_t /*workspace_bytes*/,
+                             float alpha, unsigned flags, void* workspace, size_t workspace_bytes,
                              void* stream)
 {
     const ConvPlan* pl = (const ConvPlan*)plan;
@@ -197,17 +201,18 @@ extern "C" int ng_conv_fprop(const void* plan, int in_dtype, const void* I, cons
     int rc;
     if ((rc = check_ptr16(I, "I")) || (rc = check_ptr16(F, "F")) || (rc = check_ptr16(O, "O"))) return rc;
     hipStream_t st = (hipStream_t)stream;
+    if ((uintptr_t)workspace & 15) { workspace = nullptr; workspace_bytes = 0; }   // optional here: only small grids slice
     const bool blocked = pl->fprop_blocked;
     if (pl->dtype == NG_F16) {
         if (in_dtype == NG_F16)
-            return blocked ? fprop_h<_Float16, true>(*pl, I, F, O, alpha, flags, st)
-                           : fprop_h<_Float16, false>(*pl, I, F, O, alpha, flags, st);
+            return blocked ? fprop_h<_Float16, true>(*pl, I, F, O, alpha, flags, st, workspace, workspace_bytes)
+                           : fprop_h<_Float16, false>(*pl, I, F, O, alpha, flags, st, workspace, workspace_bytes);
         // byte inputs: first layers, few channels
-        if (in_dtype == NG_U8) return fprop_h<u8_t, false>(*pl, I, F, O, alpha, flags, st);
-        if (in_dtype == NG_I8) return fprop_h<s8_t, false>(*pl, I, F, O, alpha, flags, st);
+        if (in_dtype == NG_U8) return fprop_h<u8_t, false>(*pl, I, F, O, alpha, flags, st, workspace, workspace_bytes);
+        if (in_dtype == NG_I8) return fprop_h<s8_t, false>(*pl, I, F, O, alpha, flags, st, workspace, workspace_bytes);
     } else if (in_dtype == NG_F32) {
-        return blocked ? fprop_tile<float, float, true, 128, 128, 16, 2, 2>(*pl, I, F, O, alpha, flags, st)
-                       : fprop_tile<float, float, false, 128, 128, 16, 2, 2>(*pl, I, F, O, alpha, flags, st);
+        return blocked ? fprop_tile<float, float, true, 128, 128, 16, 2, 2>(*pl, I, F, O, alpha, flags, st, 0, -1, workspace, workspace_bytes)
+                       : fprop_tile<float, float, false, 128, 128, 16, 2, 2>(*pl, I, F, O, alpha, flags, st, 0, -1, workspace, workspace_bytes);
     }
     return fail(-49, "conv fprop: unsupported input dtype %d for filter dtype %d", in_dtype, pl->dtype);
 }

@@ -47,6 +47,7 @@ struct ConvPlan {
     TapEntry* d_merged_taps = nullptr;  // m_taps entries
     TapEntry* d_merged_flat = nullptr;  // m_taps * K entries, rows (offset, k)
     size_t ws_bprop = 0, ws_update = 0;
+    size_t ws_small = 0;                // contraction slices of small forward / data-gradient grids
 };
 
 inline int cdiv(int a, int b) { return (a + b - 1) / b; }
@@ -132,6 +133,19 @@ inline int tail_column_tiles(int tiles_m, int tiles_n)
     return (rem > 0 && 4 * rem <= cus) ? rem : 0;
 }
 
+// Contraction slices for a forward / data-gradient grid that covers less than half of the
+// chip (7x7 maps: 25-75 workgroups on 256 CUs): as many as fill the chip once, each
+// keeping at least 8 contraction tiles; 1 = no slicing.
+inline int small_grid_splits(int tiles, int k_tiles, size_t slice_bytes, const void* ws, size_t ws_bytes)
+{
+    const int cus = device_cu_count();
+    if (!ws || 2 * tiles > cus || k_tiles < 16 || slice_bytes == 0) return 1;
+    int splits = std::min(cus / tiles, k_tiles / 8);
+    splits = (int)std::min<size_t>((size_t)splits, ws_bytes / slice_bytes);
+    while (splits > 1 && (splits - 1) * cdiv(k_tiles, splits) >= k_tiles) splits--;
+    return std::max(splits, 1);
+}
+
 // col_begin / col_end: the column range this launch covers (multiples of BN; default: all)
 template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, int NSTAGE = 2, class AL, class BL, class Epi>
 inline int launch_core(const AL& al, const BL& bl, const Epi& epi, int rows, int ncols, int k_tiles, int splits,
@@ -146,6 +160,23 @@ inline int launch_core(const AL& al, const BL& bl, const Epi& epi, int rows, int
     s.tiles_n = cdiv(col_end - col_begin, BN);
     s.n_base = col_begin;
     launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB, NSTAGE>(dim3(grid_tiles(s.tiles_m * s.tiles_n, splits), grid_slices(s.tiles_m * s.tiles_n, splits), 1), stream, al, bl, epi, s);
+    NG_CHECK_LAUNCH(what);
+    return 0;
+}
+
+// launch_core over the whole problem, with the contraction sliced (fp32 partial sums in `ws`,
+// added in slice order by the reduce kernel, which then runs `epi`) when the grid is small
+template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, int NSTAGE = 2, class AL, class BL, class Epi>
+inline int launch_core_sliced(const AL& al, const BL& bl, const Epi& epi, int rows, int ncols, int k_tiles,
+                              void* ws, size_t ws_bytes, hipStream_t stream, const char* what)
+{
+    const size_t slice = (size_t)rows * ncols * sizeof(float);
+    const int splits = small_grid_splits(cdiv(rows, BM) * cdiv(ncols, BN), k_tiles, slice, ws, ws_bytes);
+    if (splits == 1) return launch_core<T, BM, BN, BK, WM, WN, LA, LB, NSTAGE>(al, bl, epi, rows, ncols, k_tiles, 1, stream, what);
+    PartialEpilogue pe{(float*)ws, rows, ncols, 1, (ncols % 8 == 0) ? 1u : 0u};
+    const int rc = launch_core<T, BM, BN, BK, WM, WN, LA, LB, NSTAGE>(al, bl, pe, rows, ncols, k_tiles, splits, stream, what);
+    if (rc) return rc;
+    launch_splitk_reduce<T, Epi>((const float*)ws, splits, 1, rows, ncols, epi, stream);
     NG_CHECK_LAUNCH(what);
     return 0;
 }

@@ -156,6 +156,28 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
         }
         pl->ws_update = splits > 1 ? align_up((size_t)splits * pl->CRST * p.K * sizeof(float), 256) : 0;
     }
+    {
+        // forward and (with the filter read in place) data gradient may slice the contraction of a
+        // grid that covers less than half of the chip: room for the most slices any tile shape asks for
+        auto room = [&](int rows, long ncols_l, int kt) {
+            if (ncols_l * rows >= (1L << 30)) return (size_t)0;
+            const int ncols = (int)ncols_l;
+            const size_t slice = (size_t)rows * ncols * sizeof(float);
+            size_t bytes = 0;
+            static const int shapes[4][2] = {{256, 256}, {128, 256}, {64, 256}, {128, 128}};
+            for (const auto& t : shapes) {
+                const int sp = small_grid_splits(cdiv(rows, t[0]) * cdiv(ncols, t[1]), kt, slice, pl, ~(size_t)0);
+                if (sp > 1) bytes = std::max(bytes, (size_t)sp * slice);
+            }
+            return bytes;
+        };
+        const int kt_f = std::max(pl->RST * cdiv(p.C, pl->bk), cdiv(pl->CRST, 16));
+        pl->ws_small = room(p.K, (long)p.M * p.P * p.Q * p.N, kt_f);
+        const bool unit = p.str_d == 1 && p.str_h == 1 && p.str_w == 1;
+        if (pl->bprop_blocked && !pl->merged && unit)
+            pl->ws_small = std::max(pl->ws_small, room(p.C, (long)p.D * p.H * p.W * p.N, pl->RST * cdiv(p.K, pl->bk)));
+        pl->ws_small = align_up(pl->ws_small, 256);
+    }
     *plan_out = pl;
     return 0;
 }
@@ -179,7 +201,7 @@ int ng_conv_plan_destroy(void* plan)
 size_t ng_conv_plan_workspace_bytes(const void* plan)
 {
     const ConvPlan* pl = (const ConvPlan*)plan;
-    return pl ? std::max(pl->ws_bprop, pl->ws_update) : 0;
+    return pl ? std::max(std::max(pl->ws_bprop, pl->ws_update), pl->ws_small) : 0;
 }
 
 }  // extern "C"

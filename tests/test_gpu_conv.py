@@ -85,6 +85,10 @@ SMALL = [
     (64, 64, 64, 1, 20, 20, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     # ... and with 65 to 128 output maps on maps of 8192 pixels or more: 128-row workgroups, two column blocks per wavefront
     (64, 128, 72, 1, 91, 91, 1, 1, 3, (0, 0, 1), (1, 1, 1)),
+    # grids much smaller than the chip with long contractions (7x7 maps): forward and data gradient cut the
+    # contraction into slices with fp32 partial sums (blocked and row-by-row forward)
+    (16, 128, 128, 1, 7, 7, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (16, 24, 64, 1, 7, 7, 1, 5, 5, (0, 2, 2), (1, 1, 1)),
     # long pixel ranges with filter rows in multiples of 192: the weight gradient's 192-row tiles
     (64, 64, 32, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     (64, 64, 96, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
@@ -380,7 +384,8 @@ def test_bprop_with_rectifier_mask(ng, dtype):
                  (64, 128, 32, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)),      # main launch + tail launch
                  (128, 32, 128, 1, 6, 8, 1, 3, 3, (0, 1, 1), (1, 1, 1)),       # shared taps, 128 images
                  (128, 64, 32, 1, 4, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1)),       # ... with padded image rows
-                 (16, 128, 64, 1, 64, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1))):      # separate taps, main + tail launch
+                 (16, 128, 64, 1, 64, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)),       # separate taps, main + tail launch
+                 (16, 128, 128, 1, 7, 7, 1, 3, 3, (0, 1, 1), (1, 1, 1))):       # sliced contraction: the mask is applied by the reduce
         if dtype == np.float32 and case in FP16_ONLY:
             continue
         layer = _layer(ng, dtype, case)
