@@ -89,12 +89,29 @@ class GemmCase(object):
         return orc.ref_dot(a, b, relu=self.relu, acc_dtype=np.float32)
 
 
-def time_gpu(ng, fn, iters=20, warmup=3):
-    """average duration in ms of fn() measured with HIP events on the launch stream"""
+SETTLE_MS = float(os.environ.get("NG_BENCH_SETTLE_MS", "60"))
+
+
+def time_gpu(ng, fn, iters=20, warmup=3, settle_ms=None):
+    """average duration in ms of fn() measured with HIP events on the launch stream.
+    After an idle spell (the host preparing a case) the chip takes tens of
+    milliseconds of work to reach its sustained clocks: the same kernel measured
+    eight times in a row runs up to 18 % faster in the last measurement than in
+    the first.  The untimed part therefore lasts at least `settle_ms` of GPU time
+    (a pilot of `warmup` launches sizes it), so that what is timed is the
+    sustained rate."""
     from nervanagpu_amd import _lib
+    settle_ms = SETTLE_MS if settle_ms is None else settle_ms
+    start, end = _lib.Event(), _lib.Event()
+    warmup = max(warmup, 1)
+    start.record(ng.stream)
     for _ in range(warmup):
         fn()
-    start, end = _lib.Event(), _lib.Event()
+    end.record(ng.stream)
+    end.synchronize()
+    pilot = max(end.time_since(start) / warmup, 1e-3)
+    for _ in range(min(int(settle_ms / pilot), 20000)):
+        fn()
     start.record(ng.stream)
     for _ in range(iters):
         fn()
@@ -558,8 +575,9 @@ def mfma_ceiling(ng):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=60,
+                    help="untimed steps (a step is about 1 ms; the chip needs tens of ms to reach its sustained clocks)")
     ap.add_argument("--all", action="store_true", help="print the per-case table (stderr, or --out FILE)")
     ap.add_argument("--out", default=None, help="file for the per-case table")
     ap.add_argument("--no-cases", action="store_true", help="only the headline step, no per-case rows")

@@ -196,11 +196,12 @@ def build_network(ng, confs, dtype, zeros=False, seed=0, fold_relu=False):
     return layers
 
 
-def run_network(ng, name, dtype, loops=10, zeros=False, verbose=True, out=sys.stdout, fold_relu=False):
+def run_network(ng, name, dtype, loops=10, zeros=False, verbose=True, out=sys.stdout, fold_relu=False, warmup=None):
     net = _NETS[name]
     layers = build_network(ng, network_config(name), dtype, zeros=zeros, fold_relu=fold_relu)
     start, end = _lib.Event(), _lib.Event()
-    warmup = net["warmup"]
+    # untimed iterations: the reference's count unless the caller asks for more (sustained clocks)
+    warmup = net["warmup"] if warmup is None else max(int(warmup), net["warmup"])
     fprop_ms = bprop_ms = 0.0
     fprop_flops = bprop_flops = 0
     for loop in range(loops + warmup):
@@ -251,6 +252,8 @@ def main(argv=None):
     ap.add_argument("--nets", default="Alexnet,Overfeat,VGG,VGG_E")
     ap.add_argument("--dtypes", default="f16,f32")
     ap.add_argument("--loops", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=None,
+                    help="untimed iterations before the timed ones (default: the reference's 1, Alexnet 5)")
     ap.add_argument("--zeros", action="store_true", help="all-zero data and weights")
     ap.add_argument("--quiet", action="store_true", help="only the per-network summary")
     ap.add_argument("--json", default=None, help="write the summaries to this file")
@@ -268,7 +271,7 @@ def main(argv=None):
             print("------------------------------------------------")
             print("Benchmarking: " + title)
             print("------------------------------------------------")
-            r = run_network(ng, name, dtypes[d], loops=args.loops, zeros=args.zeros, verbose=not args.quiet,
+            r = run_network(ng, name, dtypes[d], loops=args.loops, zeros=args.zeros, verbose=not args.quiet, warmup=args.warmup,
                             fold_relu=args.fold_relu)
             results.append(r)
             print("---------------------------------------------")
