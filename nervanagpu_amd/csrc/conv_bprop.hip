@@ -343,6 +343,14 @@ extern "C" int ng_conv_bprop(const void* plan, const void* F, const void* E, voi
         (pl->ws_bprop && (rc = check_ptr16(workspace, "workspace"))))
         return rc;
     hipStream_t st = (hipStream_t)stream;
+    if (pl->pointwise && !relu_mask) {
+        // gradI (C x columns) = F (C x K) * E (K x columns)
+        const ng_conv_params& p = pl->p;
+        const int cols = p.M * p.P * p.Q * p.N;
+        const bool ws_ok = ((uintptr_t)workspace & 15) == 0;
+        return ng_gemm(pl->dtype, 0, 0, p.C, cols, p.K, F, p.K, E, cols, gradI, cols, alpha, 0.0f, 0u, 0u, 0u,
+                       1, 0, 0, 0, 1, ws_ok ? workspace : nullptr, ws_ok ? workspace_bytes : 0, stream);
+    }
     if (pl->dtype == NG_F16) return run_bprop<_Float16>(*pl, F, E, gradI, alpha, relu_mask, workspace, workspace_bytes, st);
     return run_bprop<float>(*pl, F, E, gradI, alpha, relu_mask, workspace, workspace_bytes, st);
 }

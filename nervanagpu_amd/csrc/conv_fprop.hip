@@ -202,6 +202,14 @@ extern "C" int ng_conv_fprop(const void* plan, int in_dtype, const void* I, cons
     if ((rc = check_ptr16(I, "I")) || (rc = check_ptr16(F, "F")) || (rc = check_ptr16(O, "O"))) return rc;
     hipStream_t st = (hipStream_t)stream;
     if ((uintptr_t)workspace & 15) { workspace = nullptr; workspace_bytes = 0; }   // optional here: only small grids slice
+    if (pl->pointwise && in_dtype == pl->dtype) {
+        // O (K x columns) = F^T (F is C x K) * I (C x columns): the GEMM dispatcher has the tile rules for
+        // short contractions and small outputs (832 -> 256 maps on 7x7, N = 128: 17.5 -> 8.5 us)
+        const ng_conv_params& p = pl->p;
+        const int cols = p.M * p.P * p.Q * p.N;
+        return ng_gemm(pl->dtype, 1, 0, p.K, cols, p.C, F, p.K, I, cols, O, cols, alpha, 0.0f, flags & NG_FLAG_RELU, 0u, 0u,
+                       1, 0, 0, 0, 1, workspace, workspace_bytes, stream);
+    }
     const bool blocked = pl->fprop_blocked;
     if (pl->dtype == NG_F16) {
         if (in_dtype == NG_F16)

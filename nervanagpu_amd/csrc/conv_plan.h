@@ -48,6 +48,9 @@ struct ConvPlan {
     TapEntry* d_merged_flat = nullptr;  // m_taps * K entries, rows (offset, k)
     size_t ws_bprop = 0, ws_update = 0;
     size_t ws_small = 0;                // contraction slices of small forward / data-gradient grids
+    // 1x1x1 filter, unit strides, no padding: forward and data gradient are plain matrix products
+    // (O = F^T I, gradI = F E over the (pixel, n) columns) and go to the GEMM dispatcher
+    bool pointwise = false;
 };
 
 inline int cdiv(int a, int b) { return (a + b - 1) / b; }

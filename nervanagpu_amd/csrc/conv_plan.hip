@@ -176,6 +176,13 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
         const bool unit = p.str_d == 1 && p.str_h == 1 && p.str_w == 1;
         if (pl->bprop_blocked && !pl->merged && unit)
             pl->ws_small = std::max(pl->ws_small, room(p.C, (long)p.D * p.H * p.W * p.N, pl->RST * cdiv(p.K, pl->bk)));
+        pl->pointwise = pl->RST == 1 && unit && p.pad_d == 0 && p.pad_h == 0 && p.pad_w == 0 &&
+                        (long)p.M * p.P * p.Q * p.N < (1L << 31);
+        if (pl->pointwise) {
+            const int cols = p.M * p.P * p.Q * p.N;
+            pl->ws_small = std::max(pl->ws_small, ng_gemm_workspace_bytes(dtype, 1, 0, p.K, cols, p.C, 1, 1));
+            pl->ws_small = std::max(pl->ws_small, ng_gemm_workspace_bytes(dtype, 0, 0, p.C, cols, p.K, 1, 1));
+        }
         pl->ws_small = align_up(pl->ws_small, 256);
     }
     *plan_out = pl;
