@@ -70,7 +70,19 @@ inline int conv_splits(int out_tiles, int total_k_tiles, size_t slice_bytes, siz
 {
     const int cus = device_cu_count();
     if (total_k_tiles < 8) return 1;
-    int splits = std::max(1, cus * per_cu / out_tiles);
+    const int slots = cus * per_cu;
+    int splits = std::max(1, slots / out_tiles);
+    if (splits == 1 && out_tiles < slots && slice_bytes) {
+        // More than half a round of tiles but less than a whole one (144 tiles of 256x256 on 256 CUs): a
+        // few slices can still pay.  Cost in tile steps: rounds over the chip times steps per slice, plus
+        // the fp32 partial sums written and read again (at about 5 TB/s, a tile step being about 1.4 us).
+        const double step_bytes = 1.4e-6 * 5e12 / 2;
+        double best = (double)total_k_tiles;
+        for (int s = 2; s <= 6 && s * 8 <= total_k_tiles; s++) {
+            const double cost = (double)cdiv(out_tiles * s, slots) * cdiv(total_k_tiles, s) + s * (double)slice_bytes / step_bytes;
+            if (cost < best * 0.95) { best = cost; splits = s; }
+        }
+    }
     if (total_k_tiles / splits < 15) splits = std::max(1, cus / out_tiles);
     splits = std::min(splits, std::max(1, total_k_tiles / 4));
     if (slice_bytes) splits = (int)std::min<size_t>((size_t)splits, ws_bytes / slice_bytes);

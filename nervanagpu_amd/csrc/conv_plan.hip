@@ -142,17 +142,18 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
         pl->ws_bprop = 0;
     {
         const int kt = cdiv(p.M * p.P * p.Q * p.N, pl->bk);
+        const size_t upd_slice = (size_t)pl->CRST * p.K * sizeof(float);
         // the most slices any tile shape of the update dispatcher would ask for
         static const int shapes[6][2] = {{128, 128}, {256, 256}, {64, 64}, {192, 64}, {192, 128}, {128, 64}};
         int splits = 1;
         for (const auto& t : shapes)
-            splits = std::max(splits, conv_splits(cdiv(pl->CRST, t[0]) * cdiv(p.K, t[1]), kt, 0, 0, update_tiles_per_cu(t[0], t[1])));
+            splits = std::max(splits, conv_splits(cdiv(pl->CRST, t[0]) * cdiv(p.K, t[1]), kt, upd_slice, ~(size_t)0, update_tiles_per_cu(t[0], t[1])));
         // the ring kernel of filters with three horizontal taps: 64 or 192 rows (c,t,r) per tile, W + 2 positions per image row
         if (p.S == 3 && p.K <= 128) {
             const int ring_steps = p.M * p.P * (p.W + 2), CR = p.C * p.T * p.R;
-            splits = std::max(splits, conv_splits(cdiv(CR, 64), ring_steps, 0, 0, 3));
-            splits = std::max(splits, conv_splits(cdiv(CR, 192), ring_steps, 0, 0, 1));
-            splits = std::max(splits, conv_splits(cdiv(CR, 128), ring_steps, 0, 0, 1));
+            splits = std::max(splits, conv_splits(cdiv(CR, 64), ring_steps, upd_slice, ~(size_t)0, 3));
+            splits = std::max(splits, conv_splits(cdiv(CR, 192), ring_steps, upd_slice, ~(size_t)0, 1));
+            splits = std::max(splits, conv_splits(cdiv(CR, 128), ring_steps, upd_slice, ~(size_t)0, 1));
         }
         pl->ws_update = splits > 1 ? align_up((size_t)splits * pl->CRST * p.K * sizeof(float), 256) : 0;
     }
