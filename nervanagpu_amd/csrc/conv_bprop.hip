@@ -289,12 +289,14 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
             double cost, cost_plain;
             const int row_tile = pick_row_tile(p.C, p.D * p.H * cdiv(p.W, 2) * 2 * p.N, 256, &cost);
             pick_row_tile(p.C, p.D * p.H * p.W * p.N, 256, &cost_plain);
-            if (cost <= cost_plain) {
-                switch (row_tile) {
-                case 256: return bprop_shared_taps<256, 2, 4, 256, 128, 2>(pl, F, E, gradI, alpha, mask, stream);
-                case 128: return bprop_shared_taps<128, 2, 4, 256, 128, 2>(pl, F, E, gradI, alpha, mask, stream);
-                default:  break;    // 64-row tiles: the separate taps, two workgroups per CU
-                }
+            if (cost <= cost_plain && row_tile >= 128) {
+                const int ncols = p.D * p.H * cdiv(p.W, 2) * 2 * p.N;
+                const int tail = tail_column_tiles(cdiv(p.C, row_tile), cdiv(ncols, 256));
+                const int cut = tail ? (cdiv(ncols, 256) - tail) * 256 : -1;
+                const int rc = row_tile == 256 ? bprop_shared_taps<256, 2, 4, 256, 128, 2>(pl, F, E, gradI, alpha, mask, stream, 0, cut)
+                                               : bprop_shared_taps<128, 2, 4, 256, 128, 2>(pl, F, E, gradI, alpha, mask, stream, 0, cut);
+                if (rc || !tail) return rc;
+                return bprop_shared_taps<64, 2, 2, 128, 128, 2>(pl, F, E, gradI, alpha, mask, stream, cut, -1);
             }
         } else if (shares_taps(pl)) {
             const int ncols = p.D * p.H * p.W * p.N;

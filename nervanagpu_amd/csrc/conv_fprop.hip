@@ -125,12 +125,14 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
             double cost, cost_plain;
             const int row_tile = pick_row_tile(pl.p.K, ncols, 256, &cost);
             pick_row_tile(pl.p.K, pl.p.M * pl.p.P * pl.p.Q * pl.p.N, 256, &cost_plain);
-            if (cost <= cost_plain) {
-                switch (row_tile) {
-                case 256: return fprop_shared_taps<256, 2, 4, 256, 128, 2>(pl, I, F, O, alpha, flags, st);
-                case 128: return fprop_shared_taps<128, 2, 4, 256, 128, 2>(pl, I, F, O, alpha, flags, st);
-                default:  break;    // 64-row tiles: the separate taps, two workgroups per CU
-                }
+            if (cost <= cost_plain && row_tile >= 128) {
+                // trailing column tiles beyond whole rounds: 64-row tiles of one pixel behind the main launch
+                const int tail = tail_column_tiles(cdiv(pl.p.K, row_tile), cdiv(ncols, 256));
+                const int cut = tail ? (cdiv(ncols, 256) - tail) * 256 : -1;
+                const int rc = row_tile == 256 ? fprop_shared_taps<256, 2, 4, 256, 128, 2>(pl, I, F, O, alpha, flags, st, 0, cut)
+                                               : fprop_shared_taps<128, 2, 4, 256, 128, 2>(pl, I, F, O, alpha, flags, st, 0, cut);
+                if (rc || !tail) return rc;
+                return fprop_shared_taps<64, 2, 2, 128, 128, 2>(pl, I, F, O, alpha, flags, st, cut, -1);
             }
         } else if (shares_taps(pl)) {
             const int ncols = pl.p.M * pl.p.P * cdiv(pl.p.Q, 4) * 4 * pl.p.N;

@@ -136,16 +136,20 @@ inline int pick_row_tile(int rows, int ncols, int bn, double* cost_out = nullptr
 
 // A grid of one-per-CU workgroups that is a few tiles more than a whole number
 // of rounds over the chip spends a full round on those few (784 tiles on 256 CUs:
-// four rounds for 3.06).  Returns how many trailing column tiles to take out of
-// the main launch and run behind it as many small tiles that cover the chip at
-// once: the remainder, when there is a single row tile, at least one full round,
-// and the remainder is at most a quarter of the chip; else 0.
+// four rounds for 3.06; 4 x 72 = 288 tiles: two for 1.125).  Returns how many trailing
+// column tiles (all their row tiles) to take out of the main launch and run behind it as
+// many small tiles that cover the chip at once: enough to bring the main launch down to
+// whole rounds, when there is at least one full round and the remainder is at most a
+// quarter of the chip; else 0.
 inline int tail_column_tiles(int tiles_m, int tiles_n)
 {
     const int cus = device_cu_count();
-    if (tiles_m != 1 || tiles_n <= cus) return 0;
-    const int rem = tiles_n % cus;
-    return (rem > 0 && 4 * rem <= cus) ? rem : 0;
+    const long total = (long)tiles_m * tiles_n;
+    if (total <= cus) return 0;
+    const int rem = (int)(total % cus);
+    if (rem == 0 || 4 * rem > cus) return 0;
+    const int cols = cdiv(rem, tiles_m);
+    return cols < tiles_n ? cols : 0;
 }
 
 // Contraction slices for a forward / data-gradient grid that covers less than half of the

@@ -85,6 +85,12 @@ SMALL = [
     (64, 64, 64, 1, 20, 20, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     # ... and with 65 to 128 output maps on maps of 8192 pixels or more: 128-row workgroups, two column blocks per wavefront
     (64, 128, 72, 1, 91, 91, 1, 1, 3, (0, 0, 1), (1, 1, 1)),
+    # two row tiles x 144 column tiles = 288 workgroups: the 32 beyond a whole round leave the main launch as
+    # 16 column tiles and run as small tiles behind it (64 and 128 images, forward and data gradient)
+    (64, 32, 512, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (64, 512, 32, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (128, 32, 512, 1, 16, 18, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (128, 512, 32, 1, 16, 18, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     # grids much smaller than the chip with long contractions (7x7 maps): forward and data gradient cut the
     # contraction into slices with fp32 partial sums (blocked and row-by-row forward)
     (16, 128, 128, 1, 7, 7, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
@@ -104,7 +110,9 @@ FP16_ONLY = {(64, 3, 64, 1, 20, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 5, 32, 
              (128, 32, 128, 1, 5, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (128, 64, 32, 1, 4, 13, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
              (16, 64, 128, 1, 64, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (16, 128, 64, 1, 64, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
              (64, 120, 24, 1, 5, 9, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 64, 64, 1, 20, 20, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
-             (64, 128, 72, 1, 91, 91, 1, 1, 3, (0, 0, 1), (1, 1, 1))}
+             (64, 128, 72, 1, 91, 91, 1, 1, 3, (0, 0, 1), (1, 1, 1)),
+             (64, 32, 512, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 512, 32, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+             (128, 32, 512, 1, 16, 18, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (128, 512, 32, 1, 16, 18, 1, 3, 3, (0, 1, 1), (1, 1, 1))}
 
 
 def _layer(ng, dtype, case):
