@@ -14,6 +14,7 @@
 // is read once instead of once per class.  No atomics, no zero fill, fp32
 // accumulation, one rounding.
 #include "conv_plan.h"
+#include "conv_stream_taps.h"
 
 namespace ng {
 
@@ -180,6 +181,34 @@ static int bprop_shared_taps(const ConvPlan& pl, const void* F, const void* E, v
                                                       col_begin, col_end);
 }
 
+// The same layer shape with at most 64 channels and at most 64 output maps, one
+// image plane, no rectifier mask: the (mirrored) filter stays in registers and E
+// streams (conv_stream_taps.h).  KT = 3 contraction tiles per block of 32 output maps.
+template <int KT>
+static int bprop_stream_taps(const ConvPlan& pl, const void* F, const void* E, void* gradI, float alpha, hipStream_t stream)
+{
+    typedef _Float16 T;
+    constexpr int BK = 32, TAPS = 3, PX = 4;
+    const ng_conv_params& p = pl.p;
+    const int ncols = p.H * p.W * p.N;
+    ScaleStoreEpilogue<T> epi{(T*)gradI, 0, ncols, p.C, ncols, alpha, 0.0f, 0u, 0u, 0u, 0u, 1u};
+    FilterTapColsLoader<T, BK, TAPS> al{(const T*)F, p.C, p.K, pl.RST * p.K, FastDiv::make((unsigned)p.R),
+                                        FastDiv::make((unsigned)p.R), p.R, p.R};
+    RowSegStream<T> bg{(const T*)E, p.P, p.Q, p.R - 1 - p.pad_h, p.S - 1 - p.pad_w, p.P * p.Q * p.N, p.H, p.W,
+                       FastDiv::make((unsigned)p.H)};
+    launch_stream_taps<T, 64, PX, BK, 2, 4, KT, KC>(al, bg, epi, p.H * (p.W / PX), stream);
+    NG_CHECK_LAUNCH("conv bprop (resident filter, shared taps)");
+    return 0;
+}
+
+static bool streams_shared_taps(const ConvPlan& pl, const void* mask)
+{
+    const ng_conv_params& p = pl.p;
+    return !mask && shares_taps(pl) && p.N == 64 && p.C <= 64 && p.C % 8 == 0 && p.K <= 64 && p.T == 1 && p.R == 3 &&
+           p.D == 1 && p.M == 1 && p.W % 4 == 0 && p.H * (p.W / 4) >= 4 * device_cu_count() &&
+           (long)p.P * p.Q < (1L << 19) && (long)p.C * p.H * p.W * p.N < (1L << 30);
+}
+
 // Very few channels (a first layer): rows (channel, horizontal tap), see
 // FilterChannelTapLoader.  Strips of six output pixels from eight pixels of E.
 static bool thin_channels(const ConvPlan& pl, const void* mask)
@@ -298,6 +327,8 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
                 if (rc || !tail) return rc;
                 return bprop_shared_taps<64, 2, 2, 128, 128, 2>(pl, F, E, gradI, alpha, mask, stream, cut, -1);
             }
+        } else if (streams_shared_taps(pl, mask)) {
+            return p.K == 64 ? bprop_stream_taps<6>(pl, F, E, gradI, alpha, stream) : bprop_stream_taps<3>(pl, F, E, gradI, alpha, stream);
         } else if (shares_taps(pl)) {
             const int ncols = p.D * p.H * p.W * p.N;
             const int row_tile = pick_row_tile(p.C, ncols, 256);

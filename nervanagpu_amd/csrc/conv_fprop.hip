@@ -1,6 +1,7 @@
 // Convolution forward: O = round(relu?(alpha * conv(I, F))).  Replaces
 // {h,s}conv_fprop_K64_N64 (nervanagpu/nervanagpu.py:642-650, 671-734).
 #include "conv_plan.h"
+#include "conv_stream_taps.h"
 
 namespace ng {
 
@@ -102,6 +103,34 @@ static int fprop_stream(const ConvPlan& pl, const void* I, const void* F, void* 
     return 0;
 }
 
+// Three filter rows of three taps over at most 64 channels, at most 64 output maps,
+// 64 images, one image plane: the filter stays in registers and the taps of a
+// filter row share the streamed activation tile (conv_stream_taps.h).  KT = 3
+// contraction tiles (filter rows) per block of 32 channels.
+template <int KT>
+static int fprop_stream_taps(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags,
+                             hipStream_t stream)
+{
+    typedef _Float16 T;
+    constexpr int BK = 32, TAPS = 3, PX = 4;
+    const ng_conv_params& p = pl.p;
+    const int ncols = p.P * p.Q * p.N;
+    ScaleStoreEpilogue<T> epi{(T*)O, 0, ncols, p.K, ncols, alpha, 0.0f, (flags & NG_FLAG_RELU) ? 1u : 0u, 0u, 0u, 0u, 1u};
+    FilterTapRowLoader<T, BK, TAPS> al{(const T*)F, p.K, pl.RST * p.K, FastDiv::make((unsigned)p.R), p.R, p.C};
+    RowSegStream<T> bg{(const T*)I, p.H, p.W, p.pad_h, p.pad_w, p.H * p.W * p.N, p.P, p.Q, FastDiv::make((unsigned)p.P)};
+    launch_stream_taps<T, 64, PX, BK, 2, 4, KT, MC>(al, bg, epi, p.P * (p.Q / PX), stream);
+    NG_CHECK_LAUNCH("conv fprop (resident filter, shared taps)");
+    return 0;
+}
+
+static bool streams_shared_taps(const ConvPlan& pl)
+{
+    const ng_conv_params& p = pl.p;
+    return shares_taps(pl) && p.N == 64 && p.K <= 64 && p.K % 8 == 0 && p.C <= 64 && p.T == 1 && p.R == 3 &&
+           p.D == 1 && p.M == 1 && p.Q % 4 == 0 && p.P * (p.Q / 4) >= 4 * device_cu_count() &&
+           (long)p.H * p.W < (1L << 19) && (long)p.K * p.P * p.Q * p.N < (1L << 30);
+}
+
 static bool streams_columns(const ConvPlan& pl)
 {
     const ng_conv_params& p = pl.p;
@@ -113,6 +142,11 @@ template <typename TIN, bool BLOCKED>
 static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags, hipStream_t st,
                    void* ws, size_t ws_bytes)
 {
+    if constexpr (std::is_same<TIN, _Float16>::value) {
+        // whichever way the plan would read the filter otherwise
+        if (streams_shared_taps(pl))
+            return pl.p.C == 64 ? fprop_stream_taps<6>(pl, I, F, O, alpha, flags, st) : fprop_stream_taps<3>(pl, I, F, O, alpha, flags, st);
+    }
     if constexpr (BLOCKED && std::is_same<TIN, _Float16>::value) {
         if (shares_taps(pl) && pl.p.N == 32) {
             // 32 images: 128-column tiles; 128 rows on four wavefronts

@@ -98,11 +98,19 @@ SMALL = [
     # long pixel ranges with filter rows in multiples of 192: the weight gradient's 192-row tiles
     (64, 64, 32, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     (64, 64, 96, 1, 24, 24, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    # at most 64 channels and 64 output maps on maps of four column tiles per CU or more: the filter stays in
+    # registers and the activations stream (forward and data gradient); 64 and 32 channels, whole and partial
+    # shares of column tiles per workgroup, no padding (forward only: the data gradient wants W % 4 == 0)
+    (64, 64, 64, 1, 64, 64, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (64, 32, 32, 1, 40, 104, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (64, 64, 48, 1, 66, 66, 1, 3, 3, (0, 0, 0), (1, 1, 1)),
 ]
 
 
 # cases that exist for a half-precision kernel and are large
-FP16_ONLY = {(64, 3, 64, 1, 20, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 5, 32, 1, 24, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+FP16_ONLY = {(64, 64, 64, 1, 64, 64, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 32, 32, 1, 40, 104, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+             (64, 64, 48, 1, 66, 66, 1, 3, 3, (0, 0, 0), (1, 1, 1)),
+             (64, 3, 64, 1, 20, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 5, 32, 1, 24, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
              (32, 32, 128, 2, 5, 8, 2, 3, 3, (1, 1, 1), (1, 1, 1)), (32, 64, 136, 1, 6, 12, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
              (64, 32, 128, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 128, 32, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
              (128, 32, 512, 1, 10, 14, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (128, 512, 32, 1, 10, 14, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
