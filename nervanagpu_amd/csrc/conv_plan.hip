@@ -144,7 +144,7 @@ int ng_conv_plan_create(const ng_conv_params* pp, int dtype, void** plan_out)
         const int kt = cdiv(p.M * p.P * p.Q * p.N, pl->bk);
         const size_t upd_slice = (size_t)pl->CRST * p.K * sizeof(float);
         // the most slices any tile shape of the update dispatcher would ask for
-        static const int shapes[6][2] = {{128, 128}, {256, 256}, {64, 64}, {192, 64}, {192, 128}, {128, 64}};
+        static const int shapes[7][2] = {{128, 128}, {256, 256}, {64, 64}, {192, 64}, {192, 128}, {128, 64}, {128, 192}};
         int splits = 1;
         for (const auto& t : shapes)
             splits = std::max(splits, conv_splits(cdiv(pl->CRST, t[0]) * cdiv(p.K, t[1]), kt, upd_slice, ~(size_t)0, update_tiles_per_cu(t[0], t[1])));

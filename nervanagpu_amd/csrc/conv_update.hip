@@ -125,6 +125,12 @@ static int update_h(const ConvPlan& pl, const void* I, const void* E, void* grad
             // 0.190 -> 0.166 ms; at 28x28 and 55x55 pixels the 128-row tiles,
             // which cut the contraction into fewer slices, are 7-10 % faster)
             const bool rows192 = cdiv(pl.CRST, 192) * 192 <= cdiv(pl.CRST, 128) * 128 && kdim >= 4096 * 64;
+            // output maps that fill their last 128-column tile only half (192, 320): 64-column tiles
+            // output maps in odd multiples of 192 would leave a 128-column tile half empty: 192-column
+            // tiles (three column blocks per wavefront) on contractions long enough to pay for the
+            // extra slices (64 -> 192 maps, 5x5 on 27x27, N = 128: 0.083 -> 0.073 ms)
+            if (pl.p.K % 192 == 0 && pl.p.K % 128 != 0 && kdim >= 256 * 64)
+                return launch_update<_Float16, TIN, TOUT, true, 128, 192, 64, 2, 2>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
             if (pl.p.K <= 64) {
                 if (rows192) return launch_update<_Float16, TIN, TOUT, true, 192, 64, 64, 2, 2>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
                 return launch_update<_Float16, TIN, TOUT, true, 128, 64, 64, 2, 2>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
