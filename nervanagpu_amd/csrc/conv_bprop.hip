@@ -337,8 +337,8 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
             const int ncols = p.D * p.H * p.W * p.N;
             const int row_tile = pick_row_tile(p.C, ncols, 256);
             // trailing column tiles beyond whole rounds: 64x64 tiles behind the main launch
-            // 128 rows over three rounds or more of 512-column tiles: eight pixels per tile
-            if (row_tile == 128 && p.W % 8 == 0 && cdiv(ncols, 512) >= 3 * device_cu_count()) {
+            // 128 rows over a round and a half or more of 512-column tiles: eight pixels per tile
+            if (row_tile == 128 && p.W % 8 == 0 && 2 * cdiv(ncols, 512) >= 3 * device_cu_count()) {
                 const int t512 = cdiv(ncols, 512);
                 const int wtail = tail_column_tiles(cdiv(p.C, 128), t512);
                 const int wcut = wtail ? (t512 - wtail) * 512 : -1;

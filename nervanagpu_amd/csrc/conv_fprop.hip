@@ -173,10 +173,10 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
             const int row_tile = pick_row_tile(pl.p.K, ncols, 256);
             // the few column tiles beyond whole rounds of one-per-CU workgroups run
             // behind the main launch as 64x64 tiles, which cover the chip at once
-            // 128 rows over three rounds or more of 512-column tiles: eight pixels per tile (the
+            // 128 rows over a round and a half or more of 512-column tiles: eight pixels per tile (the
             // shared segment is ten wide instead of twice six) and 64 x 128 per wavefront, the
             // fragment traffic of the 256 x 256 tile (VGG conv2.2 forward 0.271 -> 0.232 ms)
-            if (row_tile == 128 && pl.p.Q % 8 == 0 && cdiv(ncols, 512) >= 3 * device_cu_count()) {
+            if (row_tile == 128 && pl.p.Q % 8 == 0 && 2 * cdiv(ncols, 512) >= 3 * device_cu_count()) {
                 const int t512 = cdiv(ncols, 512);
                 const int wtail = tail_column_tiles(cdiv(pl.p.K, 128), t512);
                 const int wcut = wtail ? (t512 - wtail) * 512 : -1;

@@ -104,7 +104,7 @@ SMALL = [
     (64, 64, 64, 1, 64, 64, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     (64, 32, 32, 1, 40, 104, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     (64, 64, 48, 1, 66, 66, 1, 3, 3, (0, 0, 0), (1, 1, 1)),
-    # 128 rows over three rounds or more of 512-column tiles (eight pixels per tile), with a tail launch: forward / data gradient
+    # 128 rows over a round and a half or more of 512-column tiles (eight pixels per tile), with a tail launch: forward / data gradient
     (64, 32, 128, 1, 80, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     (64, 128, 32, 1, 80, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     # 192 output maps: the weight gradient's 192-column tiles
