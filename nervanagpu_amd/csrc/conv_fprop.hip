@@ -223,6 +223,11 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
         }
     }
     if constexpr (BLOCKED && std::is_same<TIN, _Float16>::value) {
+        // 128 rows and more 256-column tiles than CUs: 512-column tiles, 64 x 128 per wavefront
+        if (row_tile == 128 && (long)cdiv(pl.p.K, 128) * cdiv(ncols, 256) > device_cu_count())
+            return fprop_tile<_Float16, TIN, BLOCKED, 128, 512, 64, 2, 4>(pl, I, F, O, alpha, flags, st, 0, -1, ws, ws_bytes);
+    }
+    if constexpr (BLOCKED && std::is_same<TIN, _Float16>::value) {
         // as with the shared taps: the few column tiles beyond whole rounds of one-per-CU
         // workgroups run behind the main launch as 64x64 tiles
         const int tail = row_tile >= 128 ? tail_column_tiles(cdiv(pl.p.K, row_tile), cdiv(ncols, 256)) : 0;

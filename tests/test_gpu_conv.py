@@ -107,6 +107,9 @@ SMALL = [
     # 128 rows over a round and a half or more of 512-column tiles (eight pixels per tile), with a tail launch: forward / data gradient
     (64, 32, 128, 1, 80, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     (64, 128, 32, 1, 80, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    # 128 rows on the kernels with separate taps (16 images) and more 256-column tiles than CUs: 512-column tiles
+    (16, 64, 128, 1, 72, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+    (16, 128, 64, 1, 72, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     # 192 output maps: the weight gradient's 192-column tiles
     (64, 32, 192, 1, 20, 20, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
     # output maps in multiples of 192 over more than a round of column tiles: 192-row forward tiles
@@ -126,6 +129,7 @@ FP16_ONLY = {(64, 64, 64, 1, 64, 64, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 32, 32
              (64, 32, 128, 1, 80, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 128, 32, 1, 80, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
              (64, 48, 32, 1, 64, 64, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (16, 64, 192, 1, 80, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
              (64, 32, 192, 1, 20, 20, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
+             (16, 64, 128, 1, 72, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (16, 128, 64, 1, 72, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
              (64, 3, 64, 1, 20, 80, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 5, 32, 1, 24, 72, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
              (32, 32, 128, 2, 5, 8, 2, 3, 3, (1, 1, 1), (1, 1, 1)), (32, 64, 136, 1, 6, 12, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
              (64, 32, 128, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)), (64, 128, 32, 1, 36, 32, 1, 3, 3, (0, 1, 1), (1, 1, 1)),
