@@ -555,18 +555,57 @@ def calibrate(ng, names):
                                     "cases": done}}))
 
 
+MFMA_LOOP_SOURCE = r"""
+typedef _Float16 half8_t   __attribute__((ext_vector_type(8)));
+typedef float    float16_t __attribute__((ext_vector_type(16)));
+
+// 256 threads = one wavefront per SIMD; 16 independent 32x32 accumulators per
+// wavefront, so the matrix pipe never waits on a dependency; no memory traffic
+extern "C" __global__ __launch_bounds__(256)
+void mfma_loop(float* out, int iters, int random_data)
+{
+    half8_t a, b;
+    unsigned h = (blockIdx.x * 256u + threadIdx.x) * 2654435761u + 12345u;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        h ^= h >> 15; h *= 0x2c1b3c6du; h ^= h >> 12; h *= 0x297a2d39u; h ^= h >> 15;
+        a[i] = random_data ? (_Float16)(((int)(h & 2047) - 1024) * (1.0f / 1024)) : (_Float16)1.0f;
+        b[i] = random_data ? (_Float16)(((int)((h >> 11) & 2047) - 1024) * (1.0f / 1024)) : (_Float16)0.5f;
+    }
+    float16_t acc[16];
+#pragma unroll
+    for (int j = 0; j < 16; j++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[j][v] = 0.0f;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int j = 0; j < 16; j++) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[j], 0, 0, 0);
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 16; j++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) s += acc[j][v];
+    out[blockIdx.x * 256u + threadIdx.x] = s;
+}
+"""
+
+
 def mfma_ceiling(ng):
-    """The loop of back-to-back MFMAs without memory traffic (ng_probe_mfma_loop),
-    two workgroups of four wavefronts per CU, on constant and on random operands:
-    what the matrix pipes deliver at the clock the power limit allows."""
+    """A loop of back-to-back MFMAs without memory traffic (compiled at run time
+    from MFMA_LOOP_SOURCE; a yardstick, not part of the library), two workgroups
+    of four wavefronts per CU, on constant and on random operands: what the
+    matrix pipes deliver at the clock the power limit allows."""
     import ctypes
     from nervanagpu_amd import _lib
     blocks, out = 512, {}
     buf = ng.empty((blocks, 256), dtype=np.float32)
+    kernel = _lib.Module(MFMA_LOOP_SOURCE, "mfma_loop").get_function("mfma_loop")
     for label, rnd in (("constant", 0), ("random", 1)):
         for iters in (4000, 40000):
             def run():
-                _lib.call("ng_probe_mfma_loop", blocks, iters, rnd, ctypes.c_void_p(buf.ptr), ng.stream)
+                kernel.launch((blocks, 1, 1), (256, 1, 1), ng.stream,
+                              [ctypes.c_void_p(buf.ptr), ctypes.c_int(iters), ctypes.c_int(rnd)])
             ms = time_gpu(ng, run, iters=5, warmup=1)
             out["%s operands, %d rounds (%.2f ms)" % (label, iters, ms)] = blocks * 4 * iters * 16 * 32768.0 / ms / 1e9
     print(json.dumps({"mfma_ceiling_tflops": out, "peak": PEAK_FP16_TFLOPS}))

@@ -121,26 +121,37 @@ int ng_gemm_noalloc(int dtype, int trans_a, int trans_b, int m, int n, int k,
 
 /* GEMM-only C entry compatible with kernels/C_interface/nervana_c_api.h:31-128
  * (CUstream -> hipStream_t passed as void*; rand_state is unused because the
- * random stream is counter based; `grid` is accepted and ignored). */
+ * random stream is counter based: seed 0, one stream per stochastic call,
+ * numbered from 1 in call order; `grid` is accepted and ignored, and defaults
+ * to -1 for C++ callers as at nervana_c_api.h:74,107,117,127, so the 17-argument
+ * calls of kernels/C_interface/test.cu:28,43 compile unchanged).  Shapes that
+ * fill the chip only with a sliced contraction keep their partial sums in the
+ * static array of ng_gemm_noalloc; calls on different streams that use it are
+ * ordered among themselves with an event. */
+#ifdef __cplusplus
+#define NG_GRID_DEFAULT = -1
+#else
+#define NG_GRID_DEFAULT
+#endif
 bool nervana_loadKernels(const char* base_path);
 bool nervana_unloadKernels(void);
 size_t nervana_randStateSizeBytes(void);
 bool nervana_sgemm(float* A, float* B, float* C, bool a_t, bool b_t,
                    int m, int n, int k, int lda, int ldb, int ldc,
                    float alpha, float beta, unsigned int* rand_state,
-                   bool stochastic_round, bool apply_relu, void* stream, int grid);
+                   bool stochastic_round, bool apply_relu, void* stream, int grid NG_GRID_DEFAULT);
 bool nervana_hgemm(short* A, short* B, short* C, bool a_t, bool b_t,
                    int m, int n, int k, int lda, int ldb, int ldc,
                    float alpha, float beta, unsigned int* rand_state,
-                   bool stochastic_round, bool apply_relu, void* stream, int grid);
+                   bool stochastic_round, bool apply_relu, void* stream, int grid NG_GRID_DEFAULT);
 bool nervana_sgemm_colmajor(float* A, float* B, float* C, bool a_t, bool b_t,
                             int m, int n, int k, int lda, int ldb, int ldc,
                             float alpha, float beta, unsigned int* rand_state,
-                            bool stochastic_round, bool apply_relu, void* stream, int grid);
+                            bool stochastic_round, bool apply_relu, void* stream, int grid NG_GRID_DEFAULT);
 bool nervana_hgemm_colmajor(short* A, short* B, short* C, bool a_t, bool b_t,
                             int m, int n, int k, int lda, int ldb, int ldc,
                             float alpha, float beta, unsigned int* rand_state,
-                            bool stochastic_round, bool apply_relu, void* stream, int grid);
+                            bool stochastic_round, bool apply_relu, void* stream, int grid NG_GRID_DEFAULT);
 
 /* ---- convolution ----------------------------------------------------------
  * Direct convolution in CHWN layout: I (C,D,H,W,N), F (C,T,R,S,K),
@@ -226,14 +237,6 @@ int ng_transpose(int dtype, const void* in, void* out, int rows, int cols, void*
 int ng_dimshuffle(int dtype, const void* in, void* out, int C, int TRS, int K, void* stream);
 /* dst (dtype, nearest rounding) = src (fp32) */
 int ng_fp32_convert(int dtype, const float* src, void* dst, size_t count, void* stream);
-
-/* ---- measurement probe ----------------------------------------------------------
- * No counterpart in the reference.  `blocks` workgroups of 256 threads run
- * `iters` rounds of 16 independent v_mfma_f32_32x32x16_f16 per wavefront with no
- * memory traffic (constant or pseudo-random operands) and write one float per
- * thread to `out` (blocks * 256 floats).  Flops per launch:
- * blocks * 4 * iters * 16 * 32768.  bench.py --mfma-ceiling times it. */
-int ng_probe_mfma_loop(int blocks, int iters, int random_data, float* out, void* stream);
 
 #ifdef __cplusplus
 }

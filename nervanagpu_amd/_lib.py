@@ -108,7 +108,6 @@ _SIGNATURES = {
     "ng_transpose": (c_int, [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "ng_dimshuffle": (c_int, [c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "ng_fp32_convert": (c_int, [c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
-    "ng_probe_mfma_loop": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p]),
 }
 
 EXPORTS = tuple(_SIGNATURES)

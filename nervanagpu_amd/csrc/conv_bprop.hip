@@ -301,22 +301,21 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
     // the mask shares the plain store epilogue's indexing: unit strides only
     if (mask && (pl.merged || p.str_d != 1 || p.str_h != 1 || p.str_w != 1))
         return fail(-51, "ng_conv_bprop: the rectifier mask needs unit strides");
-    // no scratch is required when the filter is read in place; an aligned one may hold contraction slices
-    if (!pl.ws_bprop && ((uintptr_t)ws & 15)) { ws = nullptr; ws_bytes = 0; }
-    if (pl.ws_bprop && (ws_bytes < pl.ws_bprop || !ws))
-        return fail(-40, "ng_conv_bprop: workspace too small (%zu < %zu)", ws_bytes, pl.ws_bprop);
-    if (pl.merged)
+    // A misaligned workspace is never used.  The re-laid-out filter needs one (merged classes, and the
+    // row-by-row kernels of layers with few output maps); the kernels that read the filter in place
+    // do not, and run without: the requirement is checked where the filter is re-laid out.
+    if ((uintptr_t)ws & 15) { ws = nullptr; ws_bytes = 0; }
+    auto require_filter_scratch = [&]() -> int {
+        if (pl.ws_bprop && (ws_bytes < pl.ws_bprop || !ws))
+            return fail(-40, "ng_conv_bprop: workspace too small (%zu < %zu)", ws_bytes, pl.ws_bprop);
+        return 0;
+    };
+    if (pl.merged) {
+        if (int rc = require_filter_scratch()) return rc;
         return (p.K % pl.bk == 0) ? run_bprop_merged<T, true>(pl, F, E, gradI, alpha, ws, stream)
                                   : run_bprop_merged<T, false>(pl, F, E, gradI, alpha, ws, stream);
-    T* Fs = (T*)ws;
-    const bool blocked = pl.bprop_blocked;
-    if (!blocked) {
-        const long total = (long)pl.RST * pl.Kpad * pl.Cpad;
-        const int blocks = (int)std::min<long>((total + 255) / 256, 4096);
-        hipLaunchKernelGGL(filter_relayout_kernel<T>, dim3(blocks), dim3(256), 0, stream,
-                           (const T*)F, Fs, pl.d_tap_dest, p.C, pl.RST, p.K, pl.Kpad, pl.Cpad);
-        NG_CHECK_LAUNCH("filter relayout");
     }
+    const bool blocked = pl.bprop_blocked;
     if constexpr (sizeof(T) == 2) {
         // at most 32 channels (a first layer among them): one block of 32 rows on four wavefronts
         // (VGG conv1.1: 0.141 ms against 0.226 with rows (channel, tap) on halo strips)
@@ -366,6 +365,17 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
             }
         }
     }
+    // the row-by-row kernels of a layer whose output maps do not fill contraction blocks read the
+    // filter as [(tap, k)][C] from scratch
+    T* Fs = (T*)ws;
+    if (!blocked) {
+        if (int rc = require_filter_scratch()) return rc;
+        const long total = (long)pl.RST * pl.Kpad * pl.Cpad;
+        const int blocks = (int)std::min<long>((total + 255) / 256, 4096);
+        hipLaunchKernelGGL(filter_relayout_kernel<T>, dim3(blocks), dim3(256), 0, stream,
+                           (const T*)F, Fs, pl.d_tap_dest, p.C, pl.RST, p.K, pl.Kpad, pl.Cpad);
+        NG_CHECK_LAUNCH("filter relayout");
+    }
     for (const BpropClass& c : pl.classes) {
         if (c.nz * c.ny * c.nx == 0) continue;
         int rc;
@@ -391,8 +401,7 @@ extern "C" int ng_conv_bprop(const void* plan, const void* F, const void* E, voi
     if (!pl) return fail(-48, "conv: null plan");
     int rc;
     if ((rc = check_ptr16(F, "F")) || (rc = check_ptr16(E, "E")) || (rc = check_ptr16(gradI, "grad_I")) ||
-        (relu_mask && (rc = check_ptr16(relu_mask, "relu_mask"))) ||
-        (pl->ws_bprop && (rc = check_ptr16(workspace, "workspace"))))
+        (relu_mask && (rc = check_ptr16(relu_mask, "relu_mask"))))
         return rc;
     hipStream_t st = (hipStream_t)stream;
     if (pl->pointwise && !relu_mask) {

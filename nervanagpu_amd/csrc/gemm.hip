@@ -5,6 +5,7 @@
 #include "gemm_core.h"
 
 #include <algorithm>
+#include <atomic>
 #include <mutex>
 
 namespace ng {
@@ -215,6 +216,11 @@ static __device__ __align__(256) unsigned char scratch[NG_GEMM_STATIC_SCRATCH_BY
 static constexpr int MAX_DEVICES = 64;
 static void* g_scratch_ptr[MAX_DEVICES];
 static std::mutex g_scratch_mutex;
+// The nervana_* entry points also put their partial sums into the array.  Their
+// callers may use several streams, so the last call that used it leaves an event
+// behind, and a call on another stream waits for that event first.
+struct ScratchOrder { hipEvent_t done; hipStream_t last; bool used; };
+static ScratchOrder g_scratch_order[MAX_DEVICES];
 
 namespace ng {
 
@@ -228,6 +234,9 @@ int gemm_static_scratch_setup(int device)
     hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
     if (!ptr) return fail(-31, "static scratch has no device address");
+    e = hipEventCreateWithFlags(&g_scratch_order[device].done, hipEventDisableTiming);
+    if (e != hipSuccess) return hip_fail(e, "hipEventCreateWithFlags(scratch order)");
+    g_scratch_order[device].used = false;
     g_scratch_ptr[device] = ptr;
     return 0;
 }
@@ -259,7 +268,7 @@ int ng_gemm_noalloc(int dtype, int trans_a, int trans_b, int m, int n, int k,
     // reads them, so nothing in the array has to start at zero
     return ng_gemm(dtype, trans_a, trans_b, m, n, k, A, lda, B, ldb, C, ldc, alpha, beta, flags, seed, rng_stream,
                    batch_grid, ldaz, ldbz, ldcz, batch_loops,
-                   need ? g_scratch_ptr[dev] : nullptr, need ? (size_t)NG_GEMM_STATIC_SCRATCH_BYTES : 0, stream);
+                   need ? g_scratch_ptr[dev] : nullptr, need, stream);
 }
 
 // ---- GEMM-only C interface (kernels/C_interface/nervana_c_api.h) -----------
@@ -280,9 +289,37 @@ static bool c_gemm(int dtype, void* A, void* B, void* C, bool a_t, bool b_t, int
                    int lda, int ldb, int ldc, float alpha, float beta, bool sr, bool relu, void* stream)
 {
     unsigned flags = (sr ? (NG_FLAG_SR | (10u << 16)) : 0u) | (relu ? NG_FLAG_RELU : 0u);
-    static unsigned call_counter = 0;
-    int rc = ng_gemm(dtype, a_t, b_t, m, n, k, A, lda, B, ldb, C, ldc, alpha, beta, flags,
-                     0u, sr ? ++call_counter : 0u, 1, 0, 0, 0, 1, nullptr, 0, stream);
+    // stochastic rounding: seed 0, one stream of random words per call, numbered
+    // from 1 in call order (the reference's per-thread state in rand_state,
+    // kernels/C_interface/nervana_c_api.h:59-61, is not reproducible)
+    static std::atomic<unsigned> call_counter{0};
+    const unsigned rng_stream = sr ? call_counter.fetch_add(1u) + 1u : 0u;
+    // Shapes that fill the chip only when their contraction is cut into slices
+    // (fully connected layers at a minibatch of 128) keep the partial sums in the
+    // static array, so this entry runs the same schedule as NervanaGPU.dot.
+    int dev = -1;
+    const size_t need = (m > 0 && n > 0 && k > 0) ? ng_gemm_workspace_bytes(dtype, a_t, b_t, m, n, k, 1, 1) : 0;
+    const bool sliced = need > 0 && need <= (size_t)NG_GEMM_STATIC_SCRATCH_BYTES &&
+                        hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < MAX_DEVICES && g_scratch_ptr[dev];
+    int rc;
+    if (sliced) {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        ScratchOrder& ord = g_scratch_order[dev];
+        hipError_t e = hipSuccess;
+        if (ord.used && ord.last != (hipStream_t)stream) e = hipStreamWaitEvent((hipStream_t)stream, ord.done, 0);
+        rc = (e != hipSuccess) ? hip_fail(e, "hipStreamWaitEvent(scratch order)")
+                               : ng_gemm(dtype, a_t, b_t, m, n, k, A, lda, B, ldb, C, ldc, alpha, beta, flags,
+                                         0u, rng_stream, 1, 0, 0, 0, 1, g_scratch_ptr[dev], need, stream);
+        if (rc == 0) {
+            e = hipEventRecord(ord.done, (hipStream_t)stream);
+            if (e != hipSuccess) rc = hip_fail(e, "hipEventRecord(scratch order)");
+            ord.last = (hipStream_t)stream;
+            ord.used = true;
+        }
+    } else {
+        rc = ng_gemm(dtype, a_t, b_t, m, n, k, A, lda, B, ldb, C, ldc, alpha, beta, flags,
+                     0u, rng_stream, 1, 0, 0, 0, 1, nullptr, 0, stream);
+    }
     if (rc) fprintf(stderr, "nervana gemm: %s\n", ng_last_error());
     return rc == 0;
 }

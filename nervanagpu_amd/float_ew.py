@@ -734,171 +734,202 @@ class _Plan(object):
     pass
 
 
+def _is_number(arg):
+    return type(arg) in (int, float) or isinstance(arg, (np.integer, np.floating))
+
+
+def _stack_traits(args, tensor_type):
+    """One look at a postfix stack: (axis, reduces, native_2d).
+
+    axis       the one axis every reduction of the stack runs along (1 without reductions);
+               a stack that reduces along two different axes, or along none, is refused
+               (nervanagpu/float_ew.py:1090-1103)
+    native_2d  the kernel has to see the operands' own rows and columns, because something in
+               the stack depends on them: a reduction, a one-hot generator, an operand that
+               broadcasts (fewer than two dimensions or a unit extent), a transposed view, a
+               fancy-index view or a view with gaps.  Otherwise every operand is just `size`
+               consecutive values (nervanagpu/float_ew.py:1104-1137)."""
+    ops = [a for a in args if type(a) is dict]
+    axes = set(a.get("axis", None) for a in ops if a["op"] in _reduction_ops)
+    if axes - set((0, 1)):
+        raise ValueError("Only reduction along an axis currently supported")
+    if len(axes) > 1:
+        raise ValueError("Reduction only allowed along one axis per kernel.")
+    reduces = bool(axes)
+    axis = axes.pop() if reduces else 1
+
+    def own_geometry(t):
+        thin = len(t.shape) < 2 or (len(t.shape) == 2 and 1 in t.shape)
+        return thin or t.is_trans or bool(t.take_array) or not t.is_contiguous
+
+    native_2d = (reduces or any(a["op"] == "onehot" for a in ops) or
+                 any(own_geometry(a) for a in args if isinstance(a, tensor_type)))
+    return axis, reduces, native_2d
+
+
+class _Extents(object):
+    """The (rows, columns) extents of the partial results while a postfix stack is walked:
+    operands push theirs, an operator replaces those of its inputs by their broadcast."""
+
+    def __init__(self):
+        self.pending = []
+        self.widest = [1, 1]       # broadcast of the last operator's inputs
+
+    def push(self, extent):
+        self.pending.append(tuple(extent))
+
+    def join(self, count):
+        joined = [1, 1]
+        for _ in range(count):
+            extent = self.pending.pop()
+            for d in (0, 1):
+                if extent[d] == joined[d] or extent[d] == 1:
+                    continue
+                if joined[d] != 1:
+                    raise TypeError("Input shape:%s not compatible" % (extent,))
+                joined[d] = extent[d]
+        self.widest = joined
+        return tuple(joined)
+
+    def collapse(self, axis):
+        """a reduction along `axis`: returns the reduced depth"""
+        extent = list(self.pending.pop())
+        depth = extent[axis]
+        extent[axis] = 1
+        self.pending.append(tuple(extent))
+        return depth
+
+
+def _kept_mantissa_bits(out):
+    """stochastic-rounding width of a store into `out` (0: nearest): True means the full
+    fp16 mantissa; clamped to [1, 10] for fp16 and [1, 15] for fp32
+    (nervanagpu/float_ew.py:1225-1237); integer outputs always round to nearest"""
+    bits = out.rounding
+    if not bits or out.dtype.kind != "f":
+        return 0
+    if bits is True:
+        bits = 10
+    cap = {np.float32: 15, np.float16: 10}.get(out.dtype.type)
+    if cap is not None:
+        bits = min(bits, cap)
+    return max(int(bits), 1)
+
+
 def analyse(args):
-    """Shape/stride/broadcast analysis of a postfix stack
-    (follows nervanagpu/float_ew.py:1058-1286).  Pure host logic: needs no GPU,
-    tensors only need .shape/.strides/.dtype/.size/.is_trans/.take_array/
-    .is_contiguous/.gpudata/.rounding."""
+    """Shape / stride / broadcast analysis of a postfix stack: what
+    call_compound_kernel works out before it asks for a kernel
+    (nervanagpu/float_ew.py:1058-1286).  Pure host logic: needs no GPU, tensors
+    only need .shape/.strides/.dtype/.size/.is_trans/.take_array/
+    .is_contiguous/.gpudata/.rounding.
+
+    Kernel arguments are numbered in order of first appearance.  The first tensor
+    of the stack is the output and always takes argument 0; if the same tensor
+    occurs again it is an input and gets an argument of its own (an in-place
+    expression reads through a const pointer, nervanagpu/float_ew.py:1145-1154).
+    Every other tensor, and every distinct constant, is passed once."""
     from .nervanagpu import GPUTensor
 
-    out = None
-    reduction = False
-    broadcast = transpose = takeop = False
-    contiguous = True
-    argminmax = False
-    axis = 1
-    for arg in args:
-        if type(arg) is dict:
-            op_name = arg["op"]
-            if op_name in _reduction_ops:
-                if op_name[0:3] == "arg":
-                    argminmax = True
-                if arg.get("axis", None) not in (0, 1):
-                    raise ValueError("Only reduction along an axis currently supported")
-                if reduction is True:
-                    if arg["axis"] != axis:
-                        raise ValueError("Reduction only allowed along one axis per kernel.")
-                else:
-                    reduction = True
-                    axis = arg["axis"]
-            elif op_name == "onehot":
-                takeop = True
-        elif isinstance(arg, GPUTensor):
-            if len(arg.shape) < 2 or (len(arg.shape) == 2 and (arg.shape[0] == 1 or arg.shape[1] == 1)):
-                broadcast = True
-            elif arg.is_trans:
-                transpose = True
-            elif arg.take_array:
-                takeop = True
-            elif not arg.is_contiguous:
-                contiguous = False
-
-    complex_op = broadcast or reduction or transpose or takeop or not contiguous
-    stride_order = 1 if axis == 1 else -1
+    axis, reduction, complex_op = _stack_traits(args, GPUTensor)
 
     plan = _Plan()
-    type_args, tensors_info = [], []
-    array_ids, const_ids = {}, {}
-    arg_cnt = op_cnt = 0
-    shape_stack = []
-    values = {}
-    onehots = []
-    onehot_pos = []
-    max_shape = [1, 1]
+    type_args = []
+    values = {}                    # kernel argument number -> what is passed there
+    slot_of_tensor, slot_of_const = {}, {}
+    out = None
+    extents = _Extents()
+    onehots, onehot_pos = [], []
     flat_size = None
     red_depth = 0
+    n_ops = 0
+
+    def geometry(t):
+        """(extent, [row stride, column stride]) as the kernel sees operand t; with
+        reductions down the columns (axis 0) rows and columns swap roles in the
+        strides, so that the kernel always walks along its second stride"""
+        if not complex_op:
+            return (1, t.size), [0, 1]
+        if len(t.shape) == 2:
+            extent = tuple(t.shape)
+            strides = [t.strides[0], t.strides[1]]
+        elif len(t.shape) < 2:
+            # 0-d / 1-d operands broadcast as a row vector
+            extent = (1, t.size)
+            strides = [0, t.strides[0] if t.strides else 0]
+        else:
+            raise ValueError("Operations that are not simple elementwise are only currently supported in 2 dimensions.")
+        if axis == 0:
+            strides.reverse()
+        # a unit extent broadcasts: never step along it
+        if extent[0] == 1:
+            strides[1 - axis] = 0
+        if extent[1] == 1:
+            strides[axis] = 0
+        return extent, strides
 
     for pos, arg in enumerate(args):
         if isinstance(arg, GPUTensor):
-            if complex_op:
-                if len(arg.shape) == 2:
-                    shape = tuple(arg.shape)
-                    strides = list(arg.strides[::stride_order])
-                elif len(arg.shape) < 2:
-                    # 0-d / 1-d operands broadcast as a row vector
-                    n = arg.size
-                    shape = (1, n)
-                    strides = [0, arg.strides[0] if arg.strides else 0][::stride_order]
-                else:
-                    raise ValueError("Operations that are not simple elementwise are only currently supported in 2 dimensions.")
-            else:
-                shape = (1, arg.size)
-                strides = [0, 1]
+            extent, strides = geometry(arg)
+            if not complex_op:
                 if flat_size is None:
                     flat_size = arg.size
                 elif flat_size != arg.size:
                     raise TypeError("Input shape:%s not compatible" % (arg.shape,))
-
-            key = id(arg)
-            first_out = out is None
-            if first_out:
+            is_out = out is None
+            if is_out:
                 out = arg
-                indx = arg_cnt
-                arg_cnt += 1
-                new = True
-            elif key in array_ids:
-                indx = array_ids[key]
-                new = False
+                slot = len(values)
             else:
-                indx = array_ids[key] = arg_cnt
-                arg_cnt += 1
-                new = True
-
-            if new:
-                if complex_op:
-                    if shape[0] == 1:
-                        strides[1 - axis] = 0
-                    if shape[1] == 1:
-                        strides[axis] = 0
-                take_axis = 0
-                take_ptr = None
+                slot = slot_of_tensor.get(id(arg))
+                if slot is None:
+                    slot = slot_of_tensor[id(arg)] = len(values)
+            if slot not in values:
+                take_axis, take_ptr = 0, None
                 if arg.take_array:
                     take_axis = (2 - arg.take_array[1]) if axis != 1 else (arg.take_array[1] + 1)
                     take_ptr = arg.take_array[0].gpudata
-                values[indx] = dict(ptr=int(arg.gpudata) if arg.gpudata is not None else 0,
+                values[slot] = dict(ptr=int(arg.gpudata) if arg.gpudata is not None else 0,
                                     rs=int(strides[0]), cs=int(strides[1]), take=take_ptr,
-                                    dtype=arg.dtype.str[1:], take_axis=take_axis, is_out=first_out,
+                                    dtype=arg.dtype.str[1:], take_axis=take_axis, is_out=is_out,
                                     itemsize=arg.dtype.itemsize, pos=pos)
-            type_args.append(("tensor", indx))
-            shape_stack.append(shape)
+            type_args.append(("tensor", slot))
+            extents.push(extent)
 
-        elif type(arg) in (int, float) or isinstance(arg, (np.integer, np.floating)):
+        elif _is_number(arg):
             val = float(arg)
-            if val in const_ids:
-                indx = const_ids[val]
-            else:
-                indx = const_ids[val] = arg_cnt
-                arg_cnt += 1
-                values[indx] = dict(const=val, pos=pos)
-            type_args.append(("const", indx))
-            shape_stack.append((1, 1))
+            slot = slot_of_const.get(val)
+            if slot is None:
+                slot = slot_of_const[val] = len(values)
+                values[slot] = dict(const=val, pos=pos)
+            type_args.append(("const", slot))
+            extents.push((1, 1))
 
         elif type(arg) is dict:
             op_name = arg["op"]
             if op_name in _float_ops:
-                max_shape = [1, 1]
-                for _ in range(_float_ops[op_name][0]):
-                    shape = shape_stack.pop()
-                    for i in range(2):
-                        if shape[i] != max_shape[i]:
-                            if shape[i] == 1 or max_shape[i] == 1:
-                                max_shape[i] = max(max_shape[i], shape[i])
-                            else:
-                                raise TypeError("Input shape:%s not compatible" % (shape,))
+                had_inputs = bool(extents.pending)
+                joined = extents.join(_float_ops[op_name][0])
                 if op_name == "assign":
-                    rounding = out.rounding
-                    if rounding:
-                        if rounding is True:
-                            rounding = 10
-                        elif out.dtype.type is np.float32:
-                            rounding = min(rounding, 15)
-                        elif out.dtype.type is np.float16:
-                            rounding = min(rounding, 10)
-                        rounding = max(int(rounding), 1)
-                        if out.dtype.kind != "f":
-                            rounding = 0   # integer outputs always round to nearest
-                    plan.rounding = int(rounding or 0)
-                    type_args.append(("assign", op_cnt, plan.rounding > 0))
+                    plan.rounding = _kept_mantissa_bits(out)
+                    type_args.append(("assign", n_ops, plan.rounding > 0))
                 elif op_name == "onehot":
                     hot_axis = arg["axis"] if axis else 1 - arg["axis"]
-                    type_args.append(("onehot", op_cnt, hot_axis, len(onehots)))
+                    type_args.append(("onehot", n_ops, hot_axis, len(onehots)))
                     onehots.append(arg["idx"].gpudata)
                     onehot_pos.append(pos)
-                    shape_stack.append(tuple(max_shape) if len(shape_stack) else (1, 1))
+                    extents.push(joined if had_inputs else (1, 1))
                 else:
-                    type_args.append((op_name, op_cnt))
-                    shape_stack.append(tuple(max_shape))
+                    type_args.append((op_name, n_ops))
+                    extents.push(joined)
             elif op_name in _reduction_ops:
-                shape = list(shape_stack.pop())
-                type_args.append((op_name, op_cnt))
-                red_depth = max(red_depth, shape[axis])
-                shape[axis] = 1
-                shape_stack.append(tuple(shape))
+                type_args.append((op_name, n_ops))
+                red_depth = max(red_depth, extents.collapse(axis))
             else:
                 raise TypeError("%s is not a valid operation" % op_name)
-            op_cnt += 1
+            n_ops += 1
         else:
             raise TypeError("args must be instance of GPUTensor, int, float, or dict (for operators)")
+
+    max_shape = extents.widest
 
     if out is None:
         raise TypeError("expression has no output tensor")

@@ -3,6 +3,8 @@ against the numpy oracle (np.dot check of benchmarks/gemm_test.py:27-70,
 all-ones known answer of benchmarks/gemm_test2.py:40-41 and
 kernels/C_interface/test.cu:27-124)."""
 import ctypes
+import os
+import subprocess
 
 import numpy as np
 import pytest
@@ -246,6 +248,86 @@ def test_batched_dot_forms(ng, dtype):
            acc_atol(X * N))
 
 
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_batched_dot_forms_minibatch_major(ng, dtype):
+    """the second layout of benchmarks/batched_dot_test.py:54-57 (Nin = False): activations (X, N, C),
+    3-D A with a transposed 2-D B, and a transposed 3-D A summed over the batch into a 2-D C"""
+    rng = np.random.default_rng(10)
+    X, nOut, nIn, N = 5, 96, 72, 32
+    W = rng.uniform(-1, 1, (nOut, nIn)).astype(dtype)
+    I = rng.uniform(-1, 1, (X, N, nIn)).astype(dtype)
+    E = rng.uniform(-1, 1, (X, N, nOut)).astype(dtype)
+    dW, dI, dE = ng.array(W, dtype=dtype), ng.array(I, dtype=dtype), ng.array(E, dtype=dtype)
+    dO = ng.empty((X, N, nOut), dtype=dtype)
+    dB = ng.empty((X, N, nIn), dtype=dtype)
+    dU = ng.empty((nOut, nIn), dtype=dtype)
+    ng.batched_dot(dI, dW.T, dO)               # fprop
+    ng.batched_dot(dE, dW, dB)                 # bprop
+    ng.batched_dot(dE.T, dI, dU)               # update: summed over the batch
+    _check(dO.get(), orc.ref_batched_dot(I, W.T), dtype, "fprop", acc_atol(nIn))
+    _check(dB.get(), orc.ref_batched_dot(E, W), dtype, "bprop", acc_atol(nOut))
+    _check(dU.get(), orc.ref_batched_dot(np.transpose(E, (0, 2, 1)), I, out_3d=False), dtype, "update",
+           acc_atol(X * N))
+
+
+def test_batched_dot_reference_scale_accumulate():
+    """batch accumulation at the reference's scale (benchmarks/batched_dot_test.py:19-23, 53: X = 100,
+    (3072, 32) operands): E (X,K,N) . I^T (X,N,C) summed over the batch into (K,C), 3200 terms per
+    output; dyadic operands, so the fp32 sums are exact in any order and the stochastic store is
+    compared bit for bit, as is a 3-D output with a stochastic store"""
+    from nervanagpu_amd import NervanaGPU
+    ngs = NervanaGPU(stochastic_round=10, seed=77)
+    rng = np.random.default_rng(13)
+    X, K, C, N = 100, 3072, 3072, 32
+    E, I = _dyadic(rng, (X, K, N)), _dyadic(rng, (X, C, N))
+    dE, dI = ngs.array(E), ngs.array(I)
+    dU = ngs.empty((K, C))
+    ngs.batched_dot(dE, dI.T, dU)
+    E2 = np.ascontiguousarray(np.transpose(E, (1, 0, 2))).reshape(K, X * N).astype(np.float32)
+    I2 = np.ascontiguousarray(np.transpose(I, (1, 0, 2))).reshape(C, X * N).astype(np.float32)
+    pre = E2 @ I2.T                                                                      # exact
+    r = orc.rand_sr16(77, ngs.rng_counter, np.arange(K * C, dtype=np.uint32)).reshape(K, C)
+    assert np.array_equal(dU.get().view(np.uint16), orc.round_stochastic_fp16(pre, 10, r).view(np.uint16))
+    # nearest rounding of the same sums
+    ngn = NervanaGPU(stochastic_round=False)
+    dUn = ngn.empty((K, C))
+    ngn.batched_dot(ngn.array(E), ngn.array(I).T, dUn)
+    assert np.array_equal(dUn.get().view(np.uint16), pre.astype(np.float16).view(np.uint16))
+    # 3-D output (one product per batch entry) with a stochastic store: the stream index runs over (z, i, j)
+    W = _dyadic(rng, (256, C))
+    dO = ngs.empty((8, 256, N))
+    ngs.batched_dot(ngs.array(W), dI[0:8], dO, relu=True)
+    pre = np.maximum(np.matmul(W.astype(np.float32)[None], I[0:8].astype(np.float32)), 0)
+    r = orc.rand_sr16(77, ngs.rng_counter, np.arange(pre.size, dtype=np.uint32)).reshape(pre.shape)
+    assert np.array_equal(dO.get().view(np.uint16), orc.round_stochastic_fp16(pre, 10, r).view(np.uint16))
+
+
+@pytest.mark.parametrize("op", ["nn", "nt", "tn"])
+def test_dot_one_round_of_128_tiles_three_stages(op):
+    """256 tiles of 128x128 on 256 CUs with 16 or more contraction tiles: the three-stage pipeline
+    (m = n = 2048); ragged k, beta and relu against the oracle, and a stochastic store bit for bit"""
+    from nervanagpu_amd import NervanaGPU
+    rng = np.random.default_rng(23)
+    ngn = NervanaGPU(stochastic_round=False)
+    m, n, k = 2048, 2048, 2056
+    A, B, dA, dB = _operands(ngn, op, m, n, k, np.float16, rng)
+    C0 = rng.uniform(-1, 1, (m, n)).astype(np.float16)
+    C = ngn.array(C0)
+    ngn.dot(dA, dB, C, alpha=0.5, beta=0.25, relu=True)
+    assert_fp16_within_ulp(C.get(), orc.ref_dot(A, B, C0, 0.5, 0.25, True), 1.0, "2048x2048x2056 %s" % op,
+                           acc_atol(0.5 * _absdot(A, B) + 0.25))
+    ngs = NervanaGPU(stochastic_round=10, seed=6)
+    k = 1032
+    A, B = _dyadic(rng, (m, k)), _dyadic(rng, (k, n))
+    dA = ngs.array(np.ascontiguousarray(A.T)).T if op[0] == "t" else ngs.array(A)
+    dB = ngs.array(np.ascontiguousarray(B.T)).T if op[1] == "t" else ngs.array(B)
+    C = ngs.empty((m, n))
+    ngs.dot(dA, dB, C)
+    pre = orc.ref_dot(A, B, acc_dtype=np.float32)
+    r = orc.rand_sr16(6, ngs.rng_counter, np.arange(m * n, dtype=np.uint32)).reshape(m, n)
+    assert np.array_equal(C.get().view(np.uint16), orc.round_stochastic_fp16(pre, 10, r).view(np.uint16))
+
+
 def test_stochastic_rounding_bit_exact(ng):
     """SR output bit-exact against the numpy restatement fed the same stream.
     Operands are small dyadic rationals so every fp32 sum is exact and the
@@ -422,6 +504,51 @@ def test_c_api_hgemm_colmajor(ng):
     assert lib.nervana_hgemm_colmajor(vp(dAt.ptr), vp(dB.ptr), vp(dC.ptr), True, False, m, n, k,
                                       k, k, m, 1.0, 0.0, None, False, False, None, -1)
     assert_fp16_within_ulp(dC.get().T, orc.ref_dot(A, B), 1.0, "hgemm colmajor tn", acc_atol(_absdot(A, B)))
+
+
+KAT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "c_api", "kat")
+
+
+def _run_kat(*args):
+    """the native caller of the C interface (tests/c_api/kat.cpp, built by build()), as a fresh process"""
+    assert os.path.exists(KAT), "tests/c_api/kat is not built: run __graft_entry__.build()"
+    done = subprocess.run([KAT] + list(args), stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=300)
+    assert done.returncode == 0, done.stdout.decode("utf-8", "replace")[-2000:]
+    return done.stdout.decode("utf-8", "replace")
+
+
+def test_c_api_native_caller_known_answers():
+    """kernels/C_interface/test.cu:27-124 compiled against include/nervana_hip.h, 17-argument calls:
+    sgemm of ones == size and hgemm of zeros == 0 for 11 sizes x {nn, nt, tn}"""
+    assert "known answers: 0 mismatches" in _run_kat()
+
+
+def test_c_api_native_caller_stochastic_rounding(tmp_path):
+    """nervana_hgemm(stochastic_round=true) from a fresh native process: seed 0 and one rounding stream
+    per call, numbered from 1; an unsliced shape, two fully-connected shapes whose partial sums go
+    through the library's static array (the second on another stream) and an nt shape, bit for bit
+    against the numpy restatement of fp32_to_fp16_rand (nervanagpu/float_ew.py:182-201)"""
+    out = str(tmp_path / "sr.bin")
+    _run_kat("sr", out)
+    raw = np.fromfile(out, dtype=np.uint8)
+    pos, call = 0, 0
+    while pos < raw.size:
+        m, n, k, a_t, b_t, relu = (int(v) for v in raw[pos:pos + 24].view(np.int32))
+        pos += 24
+        call += 1
+        A = raw[pos:pos + 2 * m * k].view(np.float16).reshape((k, m) if a_t else (m, k)); pos += 2 * m * k
+        B = raw[pos:pos + 2 * k * n].view(np.float16).reshape((n, k) if b_t else (k, n)); pos += 2 * k * n
+        C = raw[pos:pos + 2 * m * n].view(np.uint16).reshape(m, n); pos += 2 * m * n
+        A = A.T if a_t else A
+        B = B.T if b_t else B
+        pre = orc.ref_dot(A, B, relu=bool(relu), acc_dtype=np.float32)      # exact: dyadic operands
+        assert np.array_equal(pre.astype(np.float64), np.maximum(A.astype(np.float64) @ B.astype(np.float64),
+                                                                 0 if relu else -np.inf))
+        r = orc.rand_sr16(0, call, np.arange(m * n, dtype=np.uint32)).reshape(m, n)
+        exp = orc.round_stochastic_fp16(pre, 10, r)
+        assert np.array_equal(C, exp.view(np.uint16)), (call, m, n, k, a_t, b_t)
+        assert not np.array_equal(C, pre.astype(np.float16).view(np.uint16))
+    assert call == 4
 
 
 def test_error_paths(ng):

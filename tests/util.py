@@ -53,3 +53,29 @@ def assert_fp32_close(out, ref32, rel=1e-5, what=""):
     scale = max(np.abs(ref[nz]).mean() if nz.any() else 0.0, 1e-30)
     err = np.abs(out - ref).max() / scale
     assert err <= rel, "%s: max|d|/mean|ref| = %.3g > %.3g" % (what, err, rel)
+
+
+def assert_fp32_sum_close(out, ref64, abs_sum, nterms, what=""):
+    """fp32 result of a sum of `nterms` products against its float64 value.
+
+    Rounding in an fp32 accumulation chain moves a sum of n terms by at most
+    n * 2^-24 * sum|a_i b_i| whatever the order of the additions, and by about
+    sqrt(n) * 2^-24 * sum|a_i b_i| when the rounding errors are independent
+    (Higham & Mary 2019, probabilistic bound with constant 1).  The test takes
+    the square-root form, per element, with `abs_sum` = the same sum over the
+    absolute values of the operands, plus one rounding of the result; an index
+    or term mistake moves a result by the size of a term, thousands of times more.
+    Sums of at most 512 terms must also meet max|d| / mean|ref| <= 1e-5."""
+    out = np.asarray(out, dtype=np.float64)
+    ref = np.asarray(ref64, dtype=np.float64)
+    abs_sum = np.asarray(abs_sum, dtype=np.float64)
+    assert out.shape == ref.shape == abs_sum.shape, (out.shape, ref.shape, abs_sum.shape)
+    tol = np.sqrt(float(nterms)) * EPS32 * abs_sum + EPS32 * np.abs(ref)
+    err = np.abs(out - ref)
+    bad = err > tol
+    if bad.any():
+        i = np.argmax(err - tol)
+        raise AssertionError("%s: %d of %d elements beyond sqrt(n) 2^-24 sum|a||b| (worst: got %r ref %r bound %.3g)"
+                             % (what, bad.sum(), bad.size, out.flat[i], ref.flat[i], tol.flat[i]))
+    if nterms <= 512:
+        assert_fp32_close(out, ref, 1e-5, what)
