@@ -6,6 +6,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <cstdlib>
 #include <mutex>
 
 namespace ng {
@@ -41,7 +42,20 @@ static int choose_splits(int out_tiles, int total_k_tiles, size_t slice_bytes, s
     return std::max(splits, 1);
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, bool VEC, int NSTAGE = 2>
+// Slices for the minibatch-wide shapes (one column tile, long contraction), whose
+// workgroups hold a whole CU each: as many as give every CU at most one workgroup,
+// each slice at least four contraction tiles deep.  A grid of one and a half
+// workgroups per CU would take as long as one of two per CU.
+static int one_per_cu_splits(int out_tiles, int total_k_tiles, size_t slice_bytes, size_t ws_bytes)
+{
+    int splits = std::max(1, device_cu_count() / std::max(out_tiles, 1));
+    splits = std::min(splits, std::max(1, total_k_tiles / 4));
+    if (slice_bytes) splits = (int)std::min<size_t>((size_t)splits, ws_bytes / slice_bytes);
+    while (splits > 1 && (splits - 1) * ceil_div(total_k_tiles, splits) >= total_k_tiles) splits--;
+    return std::max(splits, 1);
+}
+
+template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, bool VEC, int NSTAGE = 2, int WK = 1>
 static int launch_gemm(const GemmArgs& g, unsigned sr_bits)
 {
     CoreShape s;
@@ -53,7 +67,8 @@ static int launch_gemm(const GemmArgs& g, unsigned sr_bits)
     const int zcount = g.batch_grid;
     const int out_tiles = s.tiles_m * s.tiles_n * zcount;
     const size_t slice_bytes = (size_t)zcount * g.m * g.n * sizeof(float);
-    s.splits = g.ws ? choose_splits(out_tiles, s.passes * s.k_tiles, slice_bytes, g.ws_bytes) : 1;
+    if (WK > 1) s.splits = g.ws ? one_per_cu_splits(out_tiles, s.passes * s.k_tiles, slice_bytes, g.ws_bytes) : 1;
+    else        s.splits = g.ws ? choose_splits(out_tiles, s.passes * s.k_tiles, slice_bytes, g.ws_bytes) : 1;
 
     DenseLoader<T, LA, VEC> al{(const T*)g.A, g.ldaz, g.lda, g.m, g.k};
     DenseLoader<T, LB, VEC> bl{(const T*)g.B, g.ldbz, g.ldb, g.n, g.k};
@@ -63,11 +78,11 @@ static int launch_gemm(const GemmArgs& g, unsigned sr_bits)
 
     dim3 grid(grid_tiles(s.tiles_m * s.tiles_n, s.splits), grid_slices(s.tiles_m * s.tiles_n, s.splits), zcount);
     if (s.splits == 1) {
-        launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB, NSTAGE>(grid, g.stream, al, bl, epi, s);
+        launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB, NSTAGE, WK>(grid, g.stream, al, bl, epi, s);
         NG_CHECK_LAUNCH("gemm kernel");
     } else {
         PartialEpilogue pe{(float*)g.ws, g.m, g.n, zcount, (g.n % 8 == 0) ? 1u : 0u};
-        launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB, NSTAGE>(grid, g.stream, al, bl, pe, s);
+        launch_mfma_core<T, BM, BN, BK, WM, WN, LA, LB, NSTAGE, WK>(grid, g.stream, al, bl, pe, s);
         NG_CHECK_LAUNCH("gemm split kernel");
         launch_splitk_reduce<T, ScaleStoreEpilogue<T>>((const float*)g.ws, s.splits, zcount, g.m, g.n, epi, g.stream);
         NG_CHECK_LAUNCH("gemm split reduce");
@@ -75,12 +90,12 @@ static int launch_gemm(const GemmArgs& g, unsigned sr_bits)
     return 0;
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, bool VEC, int NSTAGE = 2>
+template <typename T, int BM, int BN, int BK, int WM, int WN, bool VEC, int NSTAGE = 2, int WK = 1>
 static int launch_layout(const GemmArgs& g, unsigned sr_bits)
 {
-    if (!g.trans_a && !g.trans_b) return launch_gemm<T, BM, BN, BK, WM, WN, KC, MC, VEC, NSTAGE>(g, sr_bits);
-    if (!g.trans_a && g.trans_b)  return launch_gemm<T, BM, BN, BK, WM, WN, KC, KC, VEC, NSTAGE>(g, sr_bits);
-    return launch_gemm<T, BM, BN, BK, WM, WN, MC, MC, VEC, NSTAGE>(g, sr_bits);
+    if (!g.trans_a && !g.trans_b) return launch_gemm<T, BM, BN, BK, WM, WN, KC, MC, VEC, NSTAGE, WK>(g, sr_bits);
+    if (!g.trans_a && g.trans_b)  return launch_gemm<T, BM, BN, BK, WM, WN, KC, KC, VEC, NSTAGE, WK>(g, sr_bits);
+    return launch_gemm<T, BM, BN, BK, WM, WN, MC, MC, VEC, NSTAGE, WK>(g, sr_bits);
 }
 
 template <typename T>
@@ -125,7 +140,20 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
         if (4 * tiles128 <= 5 * cus && k_tiles >= 16) return launch_layout<_Float16, 128, 128, 64, 2, 2, true, 3>(g, sr_bits);
         return launch_layout<_Float16, 128, 128, 64, 2, 2, true>(g, sr_bits);
     }
-    if (g.n <= 128) return launch_layout<_Float16, 64, 128, 64, 2, 2, true>(g, sr_bits);
+    if (g.n <= 128) {
+        // EXPERIMENT knob (to be removed): NG_FC_CFG picks the minibatch-wide kernel
+        static const int fc_cfg = getenv("NG_FC_CFG") ? atoi(getenv("NG_FC_CFG")) : 0;
+        if (g.n > 64 && g.batch_grid == 1 && k_tiles >= 8) {
+            switch (fc_cfg) {
+            case 1: return launch_layout<_Float16, 128, 128, 64, 4, 1, true, 4, 2>(g, sr_bits);
+            case 2: return launch_layout<_Float16, 64, 128, 128, 2, 1, true, 3, 4>(g, sr_bits);
+            case 3: return launch_layout<_Float16, 128, 128, 128, 2, 1, true, 2, 4>(g, sr_bits);
+            case 4: return launch_layout<_Float16, 64, 128, 64, 2, 1, true, 4, 2>(g, sr_bits);
+            default: break;
+            }
+        }
+        return launch_layout<_Float16, 64, 128, 64, 2, 2, true>(g, sr_bits);
+    }
     // long contractions over half a chip or more of 128x128 tiles: two slices of
     // those beat the small tiles (1792x1792x4096 55 -> 42 us, 1536x1536x8192 88 -> 53 us)
     if (2 * tiles128 >= cus && k_tiles >= 48) return launch_layout<_Float16, 128, 128, 64, 2, 2, true>(g, sr_bits);
@@ -183,6 +211,9 @@ size_t ng_gemm_workspace_bytes(int dtype, int trans_a, int trans_b, int m, int n
     for (int bm : {64, 128})
         for (int bn : {64, 128})
             splits = std::max(splits, choose_splits(ceil_div(m, bm) * ceil_div(n, bn) * batch_grid, total_k, 0, 0));
+    // the minibatch-wide kernels (64-deep tiles or deeper) run one workgroup per CU
+    if (dtype == NG_F16 && n <= 128)
+        for (int bm : {64, 128}) splits = std::max(splits, one_per_cu_splits(ceil_div(m, bm) * batch_grid, total_k, 0, 0));
     if (splits <= 1) return 0;
     return (size_t)splits * batch_grid * m * n * sizeof(float);
 }

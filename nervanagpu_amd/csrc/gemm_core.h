@@ -697,6 +697,9 @@ struct SwizzledFrag<KC, Tile> {
         f.v = *reinterpret_cast<const half8_t*>(tile + (base ^ (step * 32)));
         return f;
     }
+    // the base from which load(.., step) reads k-step first + step; `first` must be a
+    // multiple of a power of two that every later `step` stays below
+    static __device__ __forceinline__ int skip(int base, int first) { return base ^ (first * 32); }
 };
 
 template <class Tile>
@@ -720,6 +723,7 @@ struct SwizzledFrag<MC, Tile> {
         f.v = __builtin_bit_cast(half8_t, both);
         return f;
     }
+    static __device__ __forceinline__ int skip(int base, int first) { return base + first * 16 * Tile::PITCH; }
 };
 
 // A operand of a kernel whose B tile serves TAPS filter taps.  A row-contiguous
@@ -771,14 +775,20 @@ __device__ __forceinline__ void buffer_load_chunk_to_lds(BufferRsrc rsrc, char* 
 
 template <int VM> struct WaitVmLgkm0 { static constexpr int IMM = (VM & 15) | ((VM >> 4) << 14) | (7 << 4); };
 
+// WK > 1: WK groups of WM x WN wavefronts share one output tile and split the
+// k-steps of every contraction tile among themselves (group g takes steps
+// g * KS / WK onwards), so a workgroup of WM * WN * WK wavefronts keeps a tile of
+// BK in flight per stage while each wavefront still owns a whole BM/WM x BN/WN
+// sub-tile.  The groups' accumulators are added through LDS, group by group in
+// a fixed order, before the epilogue, which group 0 runs.
 template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, int NSTAGE,
-          class ALoad, class BLoad, class Epi>
-__global__ __launch_bounds__(WM * WN * 64)
+          class ALoad, class BLoad, class Epi, int WK = 1>
+__global__ __launch_bounds__(WM * WN * WK * 64)
 void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
 {
     static_assert(ALoad::DIRECT && BLoad::DIRECT, "operands must be plain 16-byte buffer loads");
     static_assert(NSTAGE >= 2, "need at least two LDS stages");
-    constexpr int NT = WM * WN * 64;
+    constexpr int NT = WM * WN * WK * 64;
     constexpr int KSTEP = Elem<T>::KSTEP;
     constexpr int TAPS = LoaderTaps<BLoad>::taps;          // filter taps served by one B tile
     constexpr int TAP_COLS = LoaderTaps<BLoad>::cols;      // columns by which a tap shifts its window
@@ -792,20 +802,26 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     static_assert(TA::CHUNKS % NT == 0 && TB::CHUNKS % NT == 0, "tile chunks must divide evenly over threads");
     constexpr int TM = BM / WM / 32;
     constexpr int TN = BN / WN / 32;
-    static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % (2 * KSTEP) == 0, "bad tile shape");
+    static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % (2 * KSTEP * WK) == 0, "bad tile shape");
+    static_assert(WK == 1 || (TAPS == 1 && (WK & (WK - 1)) == 0), "the k-steps of a plain tile are split over a power of two of groups");
 
     constexpr int STAGE = TA::BYTES + TB::BYTES;
     constexpr int WTN = BN / WN;
     constexpr int EPITCH = WTN * 4 + 16;
     constexpr int EPI_BYTES = 32 * EPITCH;
-    constexpr int SMEM_BYTES = (NSTAGE * STAGE > EPI_BYTES * WM * WN) ? NSTAGE * STAGE : EPI_BYTES * WM * WN;
+    // accumulators of one group of wavefronts on their way to group 0
+    constexpr int RED_BYTES = (WK > 1) ? WM * WN * TM * TN * 16 * 64 * 4 : 0;
+    constexpr int SMEM_TILES = (NSTAGE * STAGE > EPI_BYTES * WM * WN) ? NSTAGE * STAGE : EPI_BYTES * WM * WN;
+    constexpr int SMEM_BYTES = (SMEM_TILES > RED_BYTES) ? SMEM_TILES : RED_BYTES;
     static_assert(SMEM_BYTES <= 160 * 1024, "tile stages exceed the LDS of a compute unit");
     __shared__ __attribute__((aligned(16))) char smem[SMEM_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave % WM, wn = wave / WM;
+    const int wtile = (WK > 1) ? wave % (WM * WN) : wave;     // which sub-tile of the output
+    const int wk = (WK > 1) ? wave / (WM * WN) : 0;           // which share of the k-steps
+    const int wm = wtile % WM, wn = wtile / WM;
 
     int tm, tn, split;
     if (!block_work(s, tm, tn, split)) return;
@@ -842,7 +858,7 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     int g_pass = t_begin / s.k_tiles;
     int g_kt = t_begin - g_pass * s.k_tiles;
     constexpr int KS = BK / KSTEP;              // k-steps per tap
-    constexpr int NSTEP = TAPS * KS;
+    constexpr int NSTEP = TAPS * KS / WK;       // k-steps of a tile this wavefront multiplies
     constexpr int N_CHUNKS = CPT_A + CPT_B;
     typename ALoad::Tile g_ta;
     typename BLoad::Tile g_tb;
@@ -887,14 +903,15 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
         if (PREP_AHEAD) gprep();
     };
 
-    // lane-constant fragment addresses
+    // lane-constant fragment addresses (of the first k-step this wavefront multiplies)
     int fa_base[TM], fb_base[TAPS][TN];
 #pragma unroll
-    for (int i = 0; i < TM; i++) fa_base[i] = FA::base(wm * TM + i, lane);
+    for (int i = 0; i < TM; i++) fa_base[i] = FA::skip(FA::base(wm * TM + i, lane), wk * NSTEP);
 #pragma unroll
     for (int tap = 0; tap < TAPS; tap++)
 #pragma unroll
-        for (int j = 0; j < TN; j++) fb_base[tap][j] = TA::BYTES + FB::base(wn * TN + j + tap * (TAP_COLS / 32), lane);
+        for (int j = 0; j < TN; j++)
+            fb_base[tap][j] = TA::BYTES + FB::skip(FB::base(wn * TN + j + tap * (TAP_COLS / 32), lane), wk * NSTEP);
 
     Frag<T> fa[2][TM], fb[2][TN];
     // k-step `step` of a tile: A lines 16*step .. +15; B lines 16*(step % KS) .. +15
@@ -1020,7 +1037,36 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
     }
 
     __syncthreads();
+    if constexpr (WK > 1) {
+        // add the groups' accumulators into group 0, one group at a time in group
+        // order (the order of the additions is fixed); value v of block (i, j) of a
+        // sub-tile sits at float ((sub-tile * TM * TN + i * TN + j) * 16 + v) * 64 + lane
+        float* red = reinterpret_cast<float*>(smem) + (size_t)wtile * (TM * TN * 16 * 64) + lane;
+#pragma unroll 1
+        for (int g = 1; g < WK; g++) {
+            if (wk == g) {
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+#pragma unroll
+                        for (int v = 0; v < 16; v++) red[((i * TN + j) * 16 + v) * 64] = acc[i][j][v];
+            }
+            __syncthreads();
+            if (wk == 0) {
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+#pragma unroll
+                        for (int v = 0; v < 16; v++) acc[i][j][v] += red[((i * TN + j) * 16 + v) * 64];
+            }
+            __syncthreads();
+        }
+        if (wk != 0) return;    // no barrier follows: the epilogue staging is private to a wavefront
+    }
     if constexpr (EpilogueWholeTile<Epi>::value) {
+        static_assert(WK == 1, "whole-tile epilogues run on every wavefront");
         static_assert(BM == 32 && WM == 1, "whole-tile epilogues take one block of 32 rows");
         static_assert(32 * BN * 4 <= SMEM_BYTES, "the fp32 tile must fit the LDS of the stages");
         float* g = reinterpret_cast<float*>(smem);
@@ -1035,7 +1081,7 @@ void mfma_gemm_direct_kernel(ALoad aload, BLoad bload, Epi epi, CoreShape s)
         __syncthreads();
         epi.tile(g, tid, NT, n0);
     } else {
-        char* stage = smem + wave * EPI_BYTES;
+        char* stage = smem + wtile * EPI_BYTES;
         EpilogueBands<TM, TN, WTN, EPITCH, 0>::run(acc, stage, lane, m0 + wm * (BM / WM), n0 + wn * WTN, z, split, epi);
     }
 }
@@ -1391,15 +1437,16 @@ inline void launch_splitk_reduce(const float* ws, int splits, int zcount, int m,
 // Launch the contraction core: the direct-to-LDS pipeline when both operands
 // are plain 16-byte buffer loads of 16-bit elements, the register-staged one
 // otherwise (fp32, element-wise edge handling, 8-bit inputs converted on load).
-template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, int NSTAGE = 2, class ALoad, class BLoad,
-          class Epi>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, int NSTAGE = 2, int WK = 1, class ALoad,
+          class BLoad, class Epi>
 inline void launch_mfma_core(dim3 grid, hipStream_t stream, const ALoad& al, const BLoad& bl, const Epi& epi,
                              const CoreShape& s)
 {
     if constexpr (sizeof(T) == 2 && ALoad::DIRECT && BLoad::DIRECT) {
-        hipLaunchKernelGGL((mfma_gemm_direct_kernel<T, BM, BN, BK, WM, WN, LA, LB, NSTAGE, ALoad, BLoad, Epi>), grid,
-                           dim3(WM * WN * 64), 0, stream, al, bl, epi, s);
+        hipLaunchKernelGGL((mfma_gemm_direct_kernel<T, BM, BN, BK, WM, WN, LA, LB, NSTAGE, ALoad, BLoad, Epi, WK>), grid,
+                           dim3(WM * WN * WK * 64), 0, stream, al, bl, epi, s);
     } else {
+        static_assert(WK == 1, "the register-staged kernel does not split its k-steps over wavefront groups");
         hipLaunchKernelGGL((mfma_gemm_kernel<T, BM, BN, BK, WM, WN, LA, LB, ALoad, BLoad, Epi>), grid,
                            dim3(WM * WN * 64), 0, stream, al, bl, epi, s);
     }
