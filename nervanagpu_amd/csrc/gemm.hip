@@ -3,6 +3,7 @@
 // NervanaGPU.dot / batched_dot (nervanagpu/nervanagpu.py:820-1105) and the
 // GEMM-only C interface (kernels/C_interface/nervana_c_api.h:31-128).
 #include "gemm_core.h"
+#include "stream_core.h"
 
 #include <algorithm>
 #include <atomic>
@@ -98,6 +99,52 @@ static int launch_layout(const GemmArgs& g, unsigned sr_bits)
     return launch_gemm<T, BM, BN, BK, WM, WN, MC, MC, VEC, NSTAGE, WK>(g, sr_bits);
 }
 
+// B operand of the streaming kernel for a dense "nt" product: column c of the
+// product is row c of B (n x k, contraction contiguous)
+struct DenseRowsGather {
+    const _Float16* X;
+    int ld, n, kdim;
+    struct Fixed { unsigned off; };
+    struct Col { unsigned off; };
+    __device__ __forceinline__ Fixed fixed(int k) const { return Fixed{k < kdim ? (unsigned)k * 2u : NG_OOB_OFFSET}; }
+    __device__ __forceinline__ Col col(int c) const { return Col{c < n ? (unsigned)c * (unsigned)ld * 2u : NG_OOB_OFFSET}; }
+    // both parts are below 2^31 when valid, so bit 31 of the sum flags an invalid part
+    __device__ __forceinline__ unsigned offset(const Fixed& f, const Col& c) const
+    {
+        return ((f.off | c.off) & NG_OOB_OFFSET) ? NG_OOB_OFFSET : f.off + c.off;
+    }
+};
+
+// "nt" products with a contraction of at most 128 (the weight gradient of a fully
+// connected layer at a minibatch of 128: m x n outputs from 128-deep rows) are
+// bound by the output stream.  64 rows of A stay in registers as MFMA fragments
+// while the rows of B run through the LDS ring of the streaming kernel, 256 output
+// columns per tile, and the stores of one tile overlap the requests of the next.
+template <int KT, bool SR>
+static int launch_nt_stream(const GemmArgs& g, unsigned sr_bits)
+{
+    typedef _Float16 T;
+    constexpr int BM = 64, BN = 256, BK = 32, WN = 4, NSTAGE = 4;
+    DenseLoader<T, KC, true> al{(const T*)g.A, 0, g.lda, g.m, g.k};
+    DenseRowsGather bg{(const T*)g.B, g.ldb, g.n, g.k};
+    ScaleStoreEpilogue<T> epi{(T*)g.C, 0, g.ldc, g.m, g.n, g.alpha, 0.0f, (g.flags & NG_FLAG_RELU) ? 1u : 0u,
+                              sr_bits, g.seed, g.rng_stream, 1u};
+    const int tiles = ceil_div(g.n, BN), row_blocks = ceil_div(g.m, BM);
+    // one workgroup per CU holds a ring of four stages: as many column groups as give every CU one
+    const int col_groups = std::max(1, std::min(tiles, device_cu_count() / row_blocks));
+    launch_stream_rows<T, BM, BN, BK, WN, KT, KC, KC, NSTAGE, SR>(al, bg, epi, tiles, row_blocks, col_groups, g.stream);
+    NG_CHECK_LAUNCH("gemm nt (streamed columns)");
+    return 0;
+}
+
+static bool nt_streams(const GemmArgs& g, unsigned sr_bits)
+{
+    return !g.trans_a && g.trans_b && g.k <= 128 && g.k > 32 && g.m >= 64 && g.n >= 1024 && g.batch_grid == 1 &&
+           g.batch_loops == 1 && g.beta == 0.0f && (sr_bits == 0u || sr_bits == 10u) &&
+           ((uintptr_t)g.C & 15) == 0 && g.ldc % 8 == 0 && g.n % 8 == 0 && (long)g.m * g.ldc < (1L << 30) &&
+           (long)g.n * g.ldb < (1L << 30) && ceil_div(g.m, 64) <= 65535;
+}
+
 template <typename T>
 static bool operands_vectorizable(const GemmArgs& g)
 {
@@ -121,6 +168,14 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
     if (!operands_vectorizable<_Float16>(g)) return launch_layout<_Float16, 128, 128, 64, 2, 2, false>(g, sr_bits);
     const int cus = device_cu_count();
     const int k_tiles = ceil_div(g.k, 64) * g.batch_loops;
+    {
+        // EXPERIMENT knob (to be removed): NG_NT_STREAM=1 enables the streamed "nt" kernel
+        static const int nt_stream = getenv("NG_NT_STREAM") ? atoi(getenv("NG_NT_STREAM")) : 0;
+        if (nt_stream && nt_streams(g, sr_bits)) {
+            if (g.k <= 64) return sr_bits ? launch_nt_stream<2, true>(g, sr_bits) : launch_nt_stream<2, false>(g, sr_bits);
+            return sr_bits ? launch_nt_stream<4, true>(g, sr_bits) : launch_nt_stream<4, false>(g, sr_bits);
+        }
+    }
     // 256x256 tiles when they cover more than half the chip and the contraction
     // is long enough to amortise their prologue and epilogue (exactly half the
     // chip is one full round of 128x128 tiles at two workgroups per CU, which is

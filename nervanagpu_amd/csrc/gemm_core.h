@@ -1217,6 +1217,30 @@ struct ScaleStoreEpilogue {
             buffer_store_chunk(rsrc, off, *reinterpret_cast<const uint4_t*>(out));
         }
     }
+    // the same store with an optional stochastic rounding at the full 10 bits (pairs of
+    // outputs share a draw): for kernels that must issue the same number of stores from
+    // every wavefront whatever the rounding mode; z is the batch index of the descriptor
+    __device__ __forceinline__ bool buffer_storable() const
+    {
+        return sizeof(bits_t) == 2 && vec && beta == 0.0f && (sr_bits == 0u || sr_bits == 10u) && mask == nullptr &&
+               fold_from == 0 && (long)m * ldc < (1L << 30);
+    }
+    __device__ __forceinline__ void store8_buffer_sr(BufferRsrc rsrc, int i, int j0, int z, const float (&acc)[8]) const
+    {
+        if constexpr (sizeof(bits_t) == 2) {
+            if (sr_bits == 0u) {
+                store8_buffer(rsrc, i, j0, acc);
+            } else {
+                const unsigned pair0 = rng_index(i, j0, z) >> 1;
+                unsigned packed[4];
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    packed[q] = ng_sr10_f16x2(scale(acc[2 * q]), scale(acc[2 * q + 1]), ng_rand32(seed, stream, pair0 + q));
+                const unsigned off = (i < m && j0 < n) ? ((unsigned)i * (unsigned)ldc + (unsigned)j0) * 2u : NG_OOB_OFFSET;
+                buffer_store_chunk(rsrc, off, *reinterpret_cast<const uint4_t*>(packed));
+            }
+        }
+    }
     __device__ __forceinline__ void store8(int i, int j0, int z, int /*split*/, const float (&acc)[8]) const
     {
         if (fold_from) {

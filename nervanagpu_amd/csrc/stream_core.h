@@ -56,11 +56,13 @@ constexpr int epilogues_in_window(int kt, int d, int kt_count)
 
 // EpilogueBands with descriptor stores: one 32-row band of a wavefront's
 // accumulators through its private LDS staging; every lane stores every piece.
-template <int TM, int TN, int WTN, int EPITCH, int I>
+// SR: the epilogue's store may round stochastically (store8_buffer_sr); row0 is the
+// first row of the workgroup's row block
+template <int TM, int TN, int WTN, int EPITCH, int I, bool SR = false>
 struct StreamBands {
     template <class Epi>
     static __device__ __forceinline__ void run(float16_t (&acc)[TM][TN], char* stage, int lane, int nbase,
-                                               BufferRsrc rsrc, const Epi& epi)
+                                               BufferRsrc rsrc, const Epi& epi, int row0 = 0)
     {
         constexpr int CPW = 32 * WTN / 8;
         static_assert(CPW % 64 == 0, "a band must be whole store instructions");
@@ -81,10 +83,11 @@ struct StreamBands {
             const float4_t lo = *reinterpret_cast<const float4_t*>(stage + r * EPITCH + cc * 4);
             const float4_t hi = *reinterpret_cast<const float4_t*>(stage + r * EPITCH + cc * 4 + 16);
             const float vals[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            epi.store8_buffer(rsrc, I * 32 + r, nbase + cc, vals);
+            if constexpr (SR) epi.store8_buffer_sr(rsrc, row0 + I * 32 + r, nbase + cc, 0, vals);
+            else              epi.store8_buffer(rsrc, row0 + I * 32 + r, nbase + cc, vals);
         }
         wave_lds_fence();
-        if constexpr (I + 1 < TM) StreamBands<TM, TN, WTN, EPITCH, I + 1>::run(acc, stage, lane, nbase, rsrc, epi);
+        if constexpr (I + 1 < TM) StreamBands<TM, TN, WTN, EPITCH, I + 1, SR>::run(acc, stage, lane, nbase, rsrc, epi, row0);
     }
 };
 
@@ -94,7 +97,15 @@ struct StreamBands {
 //   Col   col(c)         what virtual column c contributes (once per column tile)
 //   unsigned offset(Fixed, Col)   byte offset of the chunk, NG_OOB_OFFSET for zeros
 //   const T* X           the tensor
-template <typename T, int BM, int BN, int BK, int WN, int KT, int LA, int NSTAGE, class ALoad, class BGather, class Epi>
+//
+// LB: layout of the B tiles in LDS (MC: columns contiguous, the gathered activations
+// of a convolution; KC: contraction contiguous, the rows of a dense matrix).
+// gridDim.y > 1: blockIdx.y numbers blocks of BM rows of A and of the output, each
+// with its own run of workgroups along the columns (a dense product with a short
+// contraction: the rows of A stay in registers, the rows of B stream).
+// SR: the store may round stochastically (the epilogue's store8_buffer_sr).
+template <typename T, int BM, int BN, int BK, int WN, int KT, int LA, int NSTAGE, class ALoad, class BGather, class Epi,
+          int LB = MC, bool SR = false>
 __global__ __launch_bounds__(WN * 64)
 void mfma_stream_kernel(ALoad aload, BGather bg, Epi epi, int tiles)
 {
@@ -105,15 +116,16 @@ void mfma_stream_kernel(ALoad aload, BGather bg, Epi epi, int tiles)
     constexpr int KS = BK / KSTEP;
     constexpr int TM = BM / 32, TN = BN / WN / 32, WTN = BN / WN;
     using TA = SwizzledTile<T, LA, BM, BK>;
-    using TB = SwizzledTile<T, MC, BN, BK>;
+    using TB = SwizzledTile<T, LB, BN, BK>;
     using FA = SwizzledFrag<LA, TA>;
-    using FB = SwizzledFrag<MC, TB>;
+    using FB = SwizzledFrag<LB, TB>;
     constexpr int CPT_B = TB::CHUNKS / NT;
     static_assert(TB::CHUNKS % NT == 0, "B tile chunks must divide evenly over threads");
     static_assert(TA::CHUNKS % 64 == 0 && TA::BYTES <= NSTAGE * TB::BYTES, "A tile is staged through the ring, wavefront by wavefront");
     static_assert(BM % 32 == 0 && BN % (WN * 32) == 0 && BK % KSTEP == 0, "bad tile shape");
     constexpr bool WHOLE = EpilogueWholeTile<Epi>::value;
     static_assert(!WHOLE || BM == 32, "whole-tile epilogues take one block of 32 rows");
+    static_assert(!WHOLE || !SR, "whole-tile epilogues round to nearest");
     constexpr int EPITCH = WTN * 4 + 16;
     constexpr int EPI_BYTES = 32 * EPITCH;
     // a whole-tile epilogue parks its rows in the ring stage that was just multiplied
@@ -133,6 +145,7 @@ void mfma_stream_kernel(ALoad aload, BGather bg, Epi epi, int tiles)
     const int first = (int)blockIdx.x * per;
     const int count = min(per, tiles - first);
     if (count <= 0) return;
+    const int m0 = (int)blockIdx.y * BM;    // first row of this workgroup's block of A
 
     // ---- A: every contraction tile once through LDS into fragments ----
     Frag<T> fa[KT][KS][TM];
@@ -148,7 +161,7 @@ void mfma_stream_kernel(ALoad aload, BGather bg, Epi epi, int tiles)
             if (i * NT + wave * 64 < TA::CHUNKS) {   // uniform over the wavefront
                 int r, k;
                 TA::chunk_pos(tid + i * NT, r, k);
-                buffer_load_chunk_to_lds(ta.rsrc, smem + (i * NT + wave * 64) * 16, aload.offset(ta, aload.prepare(r, k)));
+                buffer_load_chunk_to_lds(ta.rsrc, smem + (i * NT + wave * 64) * 16, aload.offset(ta, aload.prepare(m0 + r, k)));
             }
         }
         __builtin_amdgcn_s_waitcnt(WaitVmLgkm0<0>::IMM);
@@ -279,7 +292,7 @@ void mfma_stream_kernel(ALoad aload, BGather bg, Epi epi, int tiles)
                     // the stage is requested into again behind the next barrier, which every
                     // thread reaches only after it has read the parked rows
                 } else {
-                    StreamBands<TM, TN, WTN, EPITCH, 0>::run(acc, smem + RING + wave * EPI_BYTES, lane, n0 + wave * WTN, out_rsrc, epi);
+                    StreamBands<TM, TN, WTN, EPITCH, 0, SR>::run(acc, smem + RING + wave * EPI_BYTES, lane, n0 + wave * WTN, out_rsrc, epi, m0);
                 }
                 clear();
             }
@@ -296,6 +309,16 @@ inline void launch_stream(const AL& al, const BG& bg, const Epi& epi, int tiles,
     const int grid = std::min(tiles, device_cu_count() * wgs_per_cu);
     hipLaunchKernelGGL((mfma_stream_kernel<T, BM, BN, BK, WN, KT, LA, NSTAGE, AL, BG, Epi>), dim3(grid), dim3(WN * 64), 0,
                        stream, al, bg, epi, tiles);
+}
+
+// the dense form: `row_blocks` blocks of BM rows (blockIdx.y), `col_groups` workgroups
+// sharing the column tiles of each
+template <typename T, int BM, int BN, int BK, int WN, int KT, int LA, int LB, int NSTAGE, bool SR, class AL, class BG, class Epi>
+inline void launch_stream_rows(const AL& al, const BG& bg, const Epi& epi, int tiles, int row_blocks, int col_groups,
+                               hipStream_t stream)
+{
+    hipLaunchKernelGGL((mfma_stream_kernel<T, BM, BN, BK, WN, KT, LA, NSTAGE, AL, BG, Epi, LB, SR>),
+                       dim3((unsigned)col_groups, (unsigned)row_blocks), dim3(WN * 64), 0, stream, al, bg, epi, tiles);
 }
 
 }  // namespace ng
