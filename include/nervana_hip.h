@@ -206,7 +206,8 @@ int ng_conv_update(const void* plan, int in_dtype, int out_dtype,
 /* ---- pooling ----------------------------------------------------------------
  * Replaces {h,s}pool_max launched by NervanaGPU._execute_pool
  * (nervanagpu/nervanagpu.py:789-818); geometry mirrors PoolLayer
- * (nervanagpu/layers.py:540-626).  op: 0 max, 1 avg. */
+ * (nervanagpu/layers.py:540-626).  op: 0 max, 1 avg, 2 l2 (square root of the sum of squares,
+ * benchmarks/pool_test.py:145-146; forward only). */
 typedef struct ng_pool_params {
     int N, C, D, H, W;
     int J, T, R, S;

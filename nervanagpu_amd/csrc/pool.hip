@@ -1,8 +1,9 @@
 // Pooling over a (J,T,R,S) window of a CHWN tensor: max and average, forward
 // and backward.  Replaces {h,s}pool_max launched by NervanaGPU._execute_pool
-// (nervanagpu/nervanagpu.py:789-818) and adds the average mode the reference
-// only names (nervanagpu/nervanagpu.py:746, numpy definition
-// benchmarks/pool_test.py:142-144).
+// (nervanagpu/nervanagpu.py:789-818) and adds the average and l2 modes the
+// reference only names (nervanagpu/nervanagpu.py:746, numpy definitions
+// benchmarks/pool_test.py:142-146; l2 = square root of the sum of squares,
+// forward only: the reference defines no derivative for it).
 //
 // These are pure streaming kernels: every thread owns VEC consecutive images
 // (16 bytes of the innermost N dimension) of one output or input element, so
@@ -102,7 +103,7 @@ struct PoolGeom {
     int relu_mask;
 };
 
-enum { OP_MAX = 0, OP_AVG = 1 };
+enum { OP_MAX = 0, OP_AVG = 1, OP_L2 = 2 };
 // argmax value no element of a window of at most 255 elements carries
 enum { NO_SLOT = 255 };
 
@@ -253,7 +254,10 @@ void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char
             for (int tap = 0; tap < NTAP; tap++) {
                 const T* e = reinterpret_cast<const T*>(&raw[tap]);
 #pragma unroll
-                for (int i = 0; i < VEC; i++) best[i] += ok[tap] ? (float)e[i] : 0.0f;
+                for (int i = 0; i < VEC; i++) {
+                    const float v = ok[tap] ? (float)e[i] : 0.0f;
+                    best[i] += (OP == OP_L2) ? v * v : v;
+                }
             }
         }
     } else {
@@ -278,7 +282,7 @@ void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char
                                 if (OP == OP_MAX) {
                                     if (v[i] > best[i]) { best[i] = v[i]; slot_of[i] = slot; }
                                 } else {
-                                    best[i] += v[i];
+                                    best[i] += (OP == OP_L2) ? v[i] * v[i] : v[i];
                                 }
                             }
                         }
@@ -299,6 +303,10 @@ void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char
             const float inv = 1.0f / (float)(g.J * g.T * g.R * g.S);
 #pragma unroll
             for (int i = 0; i < VEC; i++) best[i] *= inv;
+        }
+        if (OP == OP_L2) {
+#pragma unroll
+            for (int i = 0; i < VEC; i++) best[i] = sqrtf(best[i]);
         }
         store_vec<T, VEC>(O + o, best);
     }
@@ -635,7 +643,7 @@ static bool tiles_exactly(const ng_pool_params& p)
 static int check_params(const ng_pool_params& p, int dtype, int op)
 {
     if (dtype != NG_F16 && dtype != NG_F32) return fail(-60, "pool: dtype must be fp16 or fp32");
-    if (op != OP_MAX && op != OP_AVG) return fail(-61, "pool: op must be 0 (max) or 1 (avg)");
+    if (op != OP_MAX && op != OP_AVG && op != OP_L2) return fail(-61, "pool: op must be 0 (max), 1 (avg) or 2 (l2)");
     if (p.N <= 0 || p.C <= 0 || p.K <= 0 || p.M <= 0 || p.P <= 0 || p.Q <= 0) return fail(-62, "pool: empty geometry");
     if (p.str_j < 1 || p.str_d < 1 || p.str_h < 1 || p.str_w < 1) return fail(-63, "pool: strides must be >= 1");
     if (p.D <= 0 || p.H <= 0 || p.W <= 0) return fail(-62, "pool: empty geometry");
@@ -678,8 +686,9 @@ static int run_fprop(const ng_pool_params& p, int op, const void* I, void* O, hi
     PoolGeom g = make_geom(p, VEC, sizeof(T));
     const dim3 grid = grid_for((long)g.M * g.P * g.Q * g.nvec, g.K, g.xcd_remap);
     const int rs = square_window(p);
-    if (op == OP_MAX) launch_fprop<T, VEC, OP_MAX, false>(g, rs, grid, (const T*)I, (T*)O, nullptr, st);
-    else              launch_fprop<T, VEC, OP_AVG, false>(g, rs, grid, (const T*)I, (T*)O, nullptr, st);
+    if (op == OP_MAX)      launch_fprop<T, VEC, OP_MAX, false>(g, rs, grid, (const T*)I, (T*)O, nullptr, st);
+    else if (op == OP_AVG) launch_fprop<T, VEC, OP_AVG, false>(g, rs, grid, (const T*)I, (T*)O, nullptr, st);
+    else                   launch_fprop<T, VEC, OP_L2, false>(g, rs, grid, (const T*)I, (T*)O, nullptr, st);
     NG_CHECK_LAUNCH("pool fprop");
     return 0;
 }
@@ -797,6 +806,7 @@ int ng_pool_bprop(const ng_pool_params* p, int dtype, int op, const void* I, con
 {
     int rc = check_params(*p, dtype, op);
     if (rc) return rc;
+    if (op == OP_L2) return fail(-61, "pool bprop: l2 pooling has no backward pass (the reference defines none)");
     if (!E || !gradI || (op == OP_MAX && !I)) return fail(-66, "pool: null tensor");
     if (flags & ~(unsigned)NG_FLAG_RELU) return fail(-69, "pool bprop: unknown flag bits 0x%x", flags);
     if ((flags & NG_FLAG_RELU) && (op != OP_MAX || p->J * p->T * p->R * p->S > 255))

@@ -550,8 +550,9 @@ def _pool_windows(C, DHW, JTRS, padding, strides, KMPQ):
 
 def ref_pool_fprop(I, op, JTRS, padding=(0, 0, 0, 0), strides=None):
     """max: np.max over the window with out-of-bounds slots = -FLT_MAX;
-    avg: np.mean over all J*T*R*S slots with out-of-bounds slots = 0
-    (benchmarks/pool_test.py:38-42, 120-144).  fp32 pre-rounding value."""
+    avg: np.mean over all J*T*R*S slots with out-of-bounds slots = 0;
+    l2: sqrt of the sum of squares over the window, out-of-bounds slots = 0
+    (benchmarks/pool_test.py:38-42, 120-146).  fp32 pre-rounding value."""
     C, DHW, N, strides, KMPQ = _pool_setup(I.shape, JTRS, padding, strides)
     padv = np.finfo(np.float32).min if op == "max" else 0.0
     I2 = _slicable(np.asarray(I, dtype=np.float32), padv)
@@ -561,6 +562,8 @@ def ref_pool_fprop(I, op, JTRS, padding=(0, 0, 0, 0), strides=None):
             O[k, m, p, q, :] = np.max(I2[idx, :], axis=0)
         elif op == "avg":
             O[k, m, p, q, :] = np.mean(I2[idx, :].astype(np.float64), axis=0)
+        elif op == "l2":
+            O[k, m, p, q, :] = np.sqrt(np.sum(I2[idx, :].astype(np.float64) ** 2, axis=0))
         else:
             raise ValueError(op)
     return O

@@ -186,8 +186,31 @@ def test_config5_pool_sampled(ng):
             assert_fp16_within_ulp(B[c:c + 1], refB, 1.0, "%s bprop" % op, 1e-6)
 
 
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("case", CASES)
+def test_l2_pool_fprop(ng, dtype, case):
+    """l2 pooling (named at nervanagpu/nervanagpu.py:746, defined at benchmarks/pool_test.py:145-146):
+    the square root of the sum of squares over the window, slots outside the tensor counting as zero;
+    every geometry of the max / avg cases (unrolled 2x2 and 3x3 windows, generic loops, padding,
+    feature-map windows, the scalar path).  The reference defines no derivative: bprop refuses."""
+    layer = _layer(ng, dtype, "l2", case)
+    rng = np.random.default_rng(17)
+    I = rng.uniform(-1, 1, layer.dimI).astype(np.float16).astype(dtype)
+    dO = ng.empty(layer.dimO, dtype=dtype)
+    dO.fill(9)
+    ng.fprop_pool(layer, ng.array(I, dtype=dtype), dO)
+    ref = orc.ref_pool_fprop(I, "l2", layer.JTRS, layer.padding, layer.strides)
+    if dtype == np.float16:
+        assert_fp16_within_ulp(dO.get(), ref, 1.0, "l2 fprop", 1e-6)
+    else:
+        np.testing.assert_allclose(dO.get(), ref, rtol=1e-5, atol=1e-6)
+    with pytest.raises(ValueError):
+        ng.bprop_pool(layer, ng.empty(layer.dimI, dtype=dtype), ng.empty(layer.dimO, dtype=dtype),
+                      ng.empty(layer.dimI, dtype=dtype))
+
+
 def test_pool_errors(ng):
-    layer = ng.pool_layer(np.float16, "l2", 8, 4, 1, 6, 6, 1, 1, 2, 2)
+    layer = ng.pool_layer(np.float16, "median", 8, 4, 1, 6, 6, 1, 1, 2, 2)
     with pytest.raises(ValueError):
         ng.fprop_pool(layer, ng.empty(layer.dimI), ng.empty(layer.dimO))
     ok = ng.pool_layer(np.float16, "max", 8, 4, 1, 6, 6, 1, 1, 2, 2)

@@ -174,6 +174,26 @@ def test_pool_brute_force(case, op):
         np.testing.assert_allclose(got[i], O[w], rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("case", POOL_CASES)
+def test_l2_pool_closed_forms(case):
+    """l2 pooling (benchmarks/pool_test.py:145-146) pinned without restating it: on inputs of
+    constant magnitude c it is c * sqrt(number of window slots inside the tensor); it is positively
+    homogeneous; and its square is the window SUM of I^2, i.e. J*T*R*S times the avg pooling of I^2."""
+    C, D, H, W, N, JTRS, pad, strd = case
+    rng = np.random.default_rng(8)
+    sign = rng.choice([-1.0, 1.0], (C, D, H, W, N)).astype(np.float32)
+    inside = orc.ref_pool_fprop(np.ones_like(sign), "avg", JTRS, pad, strd) * np.prod(JTRS)   # slots inside
+    np.testing.assert_allclose(orc.ref_pool_fprop(0.75 * sign, "l2", JTRS, pad, strd), 0.75 * np.sqrt(inside), rtol=1e-6)
+    I = rng.standard_normal((C, D, H, W, N)).astype(np.float32)
+    O = orc.ref_pool_fprop(I, "l2", JTRS, pad, strd)
+    np.testing.assert_allclose(orc.ref_pool_fprop(-3.0 * I, "l2", JTRS, pad, strd), 3.0 * O, rtol=1e-6)
+    np.testing.assert_allclose(O.astype(np.float64) ** 2,
+                               orc.ref_pool_fprop(I * I, "avg", JTRS, pad, strd).astype(np.float64) * np.prod(JTRS),
+                               rtol=1e-5, atol=1e-6)
+    # a 1x1x1x1 window is the absolute value
+    np.testing.assert_allclose(orc.ref_pool_fprop(I, "l2", (1, 1, 1, 1)), np.abs(I), rtol=1e-6)
+
+
 def test_pool_against_torch():
     rng = np.random.default_rng(4)
     I = rng.standard_normal((5, 1, 12, 12, 3)).astype(np.float32)
