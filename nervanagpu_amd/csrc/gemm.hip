@@ -204,6 +204,7 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
             case 2: return launch_layout<_Float16, 64, 128, 128, 2, 1, true, 3, 4>(g, sr_bits);
             case 3: return launch_layout<_Float16, 128, 128, 128, 2, 1, true, 2, 4>(g, sr_bits);
             case 4: return launch_layout<_Float16, 64, 128, 64, 2, 1, true, 4, 2>(g, sr_bits);
+            case 6: return launch_layout<_Float16, 128, 128, 64, 2, 2, true, 4, 2>(g, sr_bits);
             default: break;
             }
         }
