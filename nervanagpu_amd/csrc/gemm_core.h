@@ -763,6 +763,10 @@ struct TapTile {
 // tile just requested before reading the current one.  Hidden from it, these
 // loads are ordered by hand: an explicit s_waitcnt vmcnt(..) precedes the
 // barrier that publishes a stage.
+// (The lane-level CPU emulation of tests/emu, which checks the index arithmetic of these
+// kernels without a GPU, supplies this one function itself: host compilers cannot take
+// the assembly.)
+#ifndef NG_HOST_EMULATION
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void buffer_load_chunk_to_lds(BufferRsrc rsrc, char* lds_base, unsigned byte_offset)
@@ -772,6 +776,7 @@ __device__ __forceinline__ void buffer_load_chunk_to_lds(BufferRsrc rsrc, char* 
                  :: "s"(lds_addr), "v"(byte_offset), "s"(rsrc) : "memory", "m0");
 }
 #pragma clang diagnostic pop
+#endif
 
 template <int VM> struct WaitVmLgkm0 { static constexpr int IMM = (VM & 15) | ((VM >> 4) << 14) | (7 << 4); };
 
