@@ -3,6 +3,8 @@
 #include "conv_plan.h"
 #include "conv_stream_taps.h"
 
+#include <cstdlib>
+
 namespace ng {
 
 template <typename T, typename TIN, bool BLOCKED, int BM, int BN, int BK, int WM, int WN, int NSTAGE = 2>
@@ -103,6 +105,39 @@ static int fprop_stream(const ConvPlan& pl, const void* I, const void* F, void* 
     return 0;
 }
 
+// First layers with large filters (7x7, 11x11 on a few channels): KT contraction tiles of 16 rows,
+// all held in registers as MFMA fragments while tiles of 512 output columns stream (see
+// TapDecodeGather).  16-deep tiles keep the padding of the last tile small (363 rows: 23 tiles).
+template <int KT>
+static int fprop_stream_rows(const ConvPlan& pl, const void* I, const void* F, void* O, float alpha, unsigned flags,
+                             hipStream_t stream)
+{
+    typedef _Float16 T;
+    constexpr int BN = 512, BK = 16;
+    const ng_conv_params& p = pl.p;
+    const int ncols = p.M * p.P * p.Q * p.N;
+    ScaleStoreEpilogue<T> epi{(T*)O, 0, ncols, p.K, ncols, alpha, 0.0f, (flags & NG_FLAG_RELU) ? 1u : 0u, 0u, 0u, 0u, 1u};
+    DenseLoader<T, MC, true> al{(const T*)F, 0, p.K, p.K, pl.CRST};
+    TapDecodeGather<T> bg{(const T*)I, pl.CRST, PixelLattice::make(p.N, ncols, p.Q, p.P * p.Q), p.str_d, p.str_h, p.str_w,
+                          p.pad_d, p.pad_h, p.pad_w, p.D, p.H, p.W, p.T, p.R, p.S,
+                          FastDiv::make((unsigned)p.S), FastDiv::make((unsigned)p.R), FastDiv::make((unsigned)p.T)};
+    // a ring of four stages of 16 KB and the epilogue staging of four wavefronts: one workgroup per CU
+    launch_stream<T, 64, BN, BK, 4, KT, MC, 4>(al, bg, epi, cdiv(ncols, BN), 1, stream);
+    NG_CHECK_LAUNCH("conv fprop (streamed columns, decoded taps)");
+    return 0;
+}
+
+// contraction tiles of the kernel above for this layer (0: it does not apply): 129 to 384
+// contraction rows (fewer run with a table entry per row), at most 64 output maps
+static int streams_decoded_taps(const ConvPlan& pl)
+{
+    const ng_conv_params& p = pl.p;
+    if (pl.fprop_blocked || p.K > 64 || p.K % 8 || p.N % 8 || pl.CRST <= 128 || pl.CRST > 384) return 0;
+    if ((long)p.M * p.P * p.Q * p.N < 512L * device_cu_count()) return 0;     // a column tile per CU or more
+    if ((long)p.C * p.D * p.H * p.W * p.N >= (1L << 30) || (long)p.K * p.M * p.P * p.Q * p.N >= (1L << 30)) return 0;
+    return cdiv(pl.CRST, 16);
+}
+
 // Three filter rows of three taps over at most 64 channels, at most 64 output maps,
 // 64 images, one image plane: the filter stays in registers and the taps of a
 // filter row share the streamed activation tile (conv_stream_taps.h).  KT = 3
@@ -199,6 +234,17 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
         }
     }
     if constexpr (!BLOCKED && std::is_same<TIN, _Float16>::value) {
+        // EXPERIMENT knob (to be removed): NG_CONV_ROWS=1 enables the filter-row streaming kernel
+        static const int tap_rows_on = getenv("NG_CONV_ROWS") ? atoi(getenv("NG_CONV_ROWS")) : 0;
+        if (tap_rows_on) {
+            // the kernel is compiled for the tile counts of the usual first layers: 7x7 on three
+            // channels (147 rows: 10 tiles), 11x11 on three channels (363 rows: 23 tiles); other
+            // counts run the next larger one with empty tiles
+            const int kt = streams_decoded_taps(pl);
+            if (kt > 0 && kt <= 10) return fprop_stream_rows<10>(pl, I, F, O, alpha, flags, st);
+            if (kt > 10 && kt <= 16) return fprop_stream_rows<16>(pl, I, F, O, alpha, flags, st);
+            if (kt > 16 && kt <= 24) return fprop_stream_rows<24>(pl, I, F, O, alpha, flags, st);
+        }
         if (streams_columns(pl)) {
             switch (cdiv(pl.CRST, 32)) {
             case 1: return fprop_stream<1>(pl, I, F, O, alpha, flags, st);

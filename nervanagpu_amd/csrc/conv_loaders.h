@@ -729,6 +729,55 @@ struct FlatTapGather {
     }
 };
 
+// Forward convolution of a first layer with a large filter (few channels, 7x7 or 11x11 taps: more
+// contraction rows than the flat gather above can keep a table entry for in registers).  What
+// contraction row j = ((c * T + t) * R + r) * S + s contributes is decoded from j itself: tile lines
+// are whole wavefront requests, so j is uniform and the three divisions run on the scalar unit; a lane
+// keeps one column descriptor per column tile, and a request costs three compares and an add.
+template <typename T>
+struct TapDecodeGather {
+    const T*     X;
+    int          J;                   // contraction rows C * T * R * S
+    PixelLattice lat;                 // output pixels (m, p, q) x n
+    int          str_d, str_h, str_w;
+    int          pad_d, pad_h, pad_w;
+    int          D, H, W;
+    int          T_, R, S;
+    FastDiv      s_div, r_div, t_div;
+    static constexpr bool FIXED_ON_DEMAND = true;
+    typedef StreamFixed Fixed;
+    typedef StreamCol Col;
+
+    __device__ __forceinline__ Fixed fixed(int j) const
+    {
+        if (j >= J) return Fixed{0, NG_FAR, NG_FAR, NG_FAR};
+        const int crt = (int)s_div.div((unsigned)j), s = j - crt * S;
+        const int ct = (int)r_div.div((unsigned)crt), r = crt - ct * R;
+        const int c = (int)t_div.div((unsigned)ct), t = ct - c * T_;
+        Fixed f;
+        f.off = __builtin_amdgcn_readfirstlane((((c * D + t) * H + r) * W + s) * lat.N);
+        f.dz = __builtin_amdgcn_readfirstlane(t);
+        f.dy = __builtin_amdgcn_readfirstlane(r);
+        f.dx = __builtin_amdgcn_readfirstlane(s);
+        return f;
+    }
+    // the origin of the column's receptive field (its first tap may lie in the padding)
+    __device__ __forceinline__ Col col(int c) const
+    {
+        if (c >= lat.ncols) return Col{0, NG_FAR, NG_FAR, NG_FAR};
+        int m, p, q, nn;
+        lat.split(c, m, p, q, nn);
+        Col o;
+        o.z0 = m * str_d - pad_d; o.y0 = p * str_h - pad_h; o.x0 = q * str_w - pad_w;
+        o.base = ((o.z0 * H + o.y0) * W + o.x0) * lat.N + nn;
+        return o;
+    }
+    __device__ __forceinline__ unsigned offset(const Fixed& f, const Col& c) const
+    {
+        return stream_offset<T>(f, c, D, H, W);
+    }
+};
+
 // data gradient with rows (channel, horizontal tap): contraction rows
 // ((t, r), output map), columns the halo strips of HaloStripLoader.
 // A line of the tile (BN = 512 columns) is exactly one wavefront request, so what

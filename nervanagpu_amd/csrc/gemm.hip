@@ -120,18 +120,19 @@ struct DenseRowsGather {
 // bound by the output stream.  64 rows of A stay in registers as MFMA fragments
 // while the rows of B run through the LDS ring of the streaming kernel, 256 output
 // columns per tile, and the stores of one tile overlap the requests of the next.
-template <int KT, bool SR>
+template <int KT, bool SR, int NSTAGE = 4, int PER_CU = 1>
 static int launch_nt_stream(const GemmArgs& g, unsigned sr_bits)
 {
     typedef _Float16 T;
-    constexpr int BM = 64, BN = 256, BK = 32, WN = 4, NSTAGE = 4;
+    constexpr int BM = 64, BN = 256, BK = 32, WN = 4;
     DenseLoader<T, KC, true> al{(const T*)g.A, 0, g.lda, g.m, g.k};
     DenseRowsGather bg{(const T*)g.B, g.ldb, g.n, g.k};
     ScaleStoreEpilogue<T> epi{(T*)g.C, 0, g.ldc, g.m, g.n, g.alpha, 0.0f, (g.flags & NG_FLAG_RELU) ? 1u : 0u,
                               sr_bits, g.seed, g.rng_stream, 1u};
     const int tiles = ceil_div(g.n, BN), row_blocks = ceil_div(g.m, BM);
-    // one workgroup per CU holds a ring of four stages: as many column groups as give every CU one
-    const int col_groups = std::max(1, std::min(tiles, device_cu_count() / row_blocks));
+    // PER_CU workgroups fit the LDS of a CU (a ring of four stages: one; of two stages: two, whose
+    // stores and stochastic rounding overlap each other's products): as many column groups as fill those slots
+    const int col_groups = std::max(1, std::min(tiles, PER_CU * device_cu_count() / row_blocks));
     launch_stream_rows<T, BM, BN, BK, WN, KT, KC, KC, NSTAGE, SR>(al, bg, epi, tiles, row_blocks, col_groups, g.stream);
     NG_CHECK_LAUNCH("gemm nt (streamed columns)");
     return 0;
@@ -173,6 +174,7 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
         static const int nt_stream = getenv("NG_NT_STREAM") ? atoi(getenv("NG_NT_STREAM")) : 0;
         if (nt_stream && nt_streams(g, sr_bits)) {
             if (g.k <= 64) return sr_bits ? launch_nt_stream<2, true>(g, sr_bits) : launch_nt_stream<2, false>(g, sr_bits);
+            if (nt_stream == 2) return sr_bits ? launch_nt_stream<4, true, 2, 2>(g, sr_bits) : launch_nt_stream<4, false, 2, 2>(g, sr_bits);
             return sr_bits ? launch_nt_stream<4, true>(g, sr_bits) : launch_nt_stream<4, false>(g, sr_bits);
         }
     }

@@ -42,6 +42,14 @@ __device__ __forceinline__ void static_for(F&& f)
 template <class G, class = void> struct GatherFixedPerTile { static constexpr bool value = false; };
 template <class G> struct GatherFixedPerTile<G, std::enable_if_t<G::FIXED_PER_TILE>> { static constexpr bool value = true; };
 
+// A gather that derives what a contraction row contributes from the row number alone, with a few
+// operations on the scalar unit, declares `static constexpr bool FIXED_ON_DEMAND = true` and
+// Fixed fixed(row), offset(Fixed, Col): nothing is kept per contraction tile, so the tiles may be
+// many (the 363 filter rows of an 11x11 first layer).  A line of its tiles must be one wavefront
+// request, so that the row is uniform.
+template <class G, class = void> struct GatherFixedOnDemand { static constexpr bool value = false; };
+template <class G> struct GatherFixedOnDemand<G, std::enable_if_t<G::FIXED_ON_DEMAND>> { static constexpr bool value = true; };
+
 template <class E, class = void> struct StoresPerThread { static constexpr int value = 0; };
 template <class E> struct StoresPerThread<E, std::enable_if_t<(E::STORES_PER_THREAD > 0)>> { static constexpr int value = E::STORES_PER_THREAD; };
 
@@ -176,15 +184,17 @@ void mfma_stream_kernel(ALoad aload, BGather bg, Epi epi, int tiles)
 
     // ---- B stream ----
     constexpr bool PER_TILE = GatherFixedPerTile<BGather>::value;
-    static_assert(!PER_TILE || TB::CPR == 64, "a tile line must be one wavefront request for its row to be uniform");
+    constexpr bool ON_DEMAND = GatherFixedOnDemand<BGather>::value;
+    static_assert(!(PER_TILE || ON_DEMAND) || TB::CPR == 64, "a tile line must be one wavefront request for its row to be uniform");
+    static_assert(!(ON_DEMAND && PER_TILE), "one or the other");
     int rc[CPT_B], kc[CPT_B];
-    typename BGather::Fixed fx[KT][PER_TILE ? 1 : CPT_B];
+    typename BGather::Fixed fx[ON_DEMAND ? 1 : KT][(PER_TILE || ON_DEMAND) ? 1 : CPT_B];
 #pragma unroll
     for (int c = 0; c < CPT_B; c++) {
         int k;
         TB::chunk_pos(tid + c * NT, rc[c], k);
-        kc[c] = PER_TILE ? __builtin_amdgcn_readfirstlane(k) : k;
-        if constexpr (!PER_TILE) {
+        kc[c] = (PER_TILE || ON_DEMAND) ? __builtin_amdgcn_readfirstlane(k) : k;
+        if constexpr (!PER_TILE && !ON_DEMAND) {
 #pragma unroll
             for (int kt = 0; kt < KT; kt++) fx[kt][c] = bg.fixed(kt * BK + k);
         }
@@ -209,7 +219,8 @@ void mfma_stream_kernel(ALoad aload, BGather bg, Epi epi, int tiles)
 #pragma unroll
                 for (int q = 0; q < KT; q++)
                     if (q == ktn) {
-                        if constexpr (PER_TILE) off = bg.offset(fx[q][0], kc[c], col[c]);
+                        if constexpr (ON_DEMAND)     off = bg.offset(bg.fixed(q * BK + kc[c]), col[c]);   // q is a constant here
+                        else if constexpr (PER_TILE) off = bg.offset(fx[q][0], kc[c], col[c]);
                         else                    off = bg.offset(fx[q][c], col[c]);
                     }
                 buffer_load_chunk_to_lds(rsrc, smem + wr_off + (c * NT + wave * 64) * 16, off);
