@@ -231,10 +231,173 @@ int device_cu_count() { return emu::g_cus; }
 
 }  // namespace ng
 
+// ---- run-time compilation: the host compiler against the same stand-in headers --------------
+#include <dlfcn.h>
+#include <unistd.h>
+
+#include <regex>
+#include <string>
+
+namespace {
+
+struct EmuModule { void* handle; std::string dir; };
+
+std::string this_library()
+{
+    Dl_info info;
+    if (dladdr((void*)&this_library, &info) && info.dli_fname) return info.dli_fname;
+    return "libnervana_emu.so";
+}
+
+std::string shim_dir()
+{
+    const std::string so = this_library();
+    const size_t slash = so.find_last_of('/');
+    return (slash == std::string::npos ? std::string(".") : so.substr(0, slash)) + "/shim";
+}
+
+// `extern "C" __global__ ... void NAME(T0 a0, T1 a1, ...)` -> a trampoline NAME__emu(void** args)
+// that unpacks the argument block of ng_launch (pointers to the values, as hipModuleLaunchKernel takes)
+std::string trampolines(const std::string& src)
+{
+    std::string out;
+    std::regex head(R"(extern\s+"C"\s+__global__[\s\S]*?void\s+(\w+)\s*\(([^\)]*)\))");
+    for (std::sregex_iterator it(src.begin(), src.end(), head), end; it != end; ++it) {
+        const std::string name = (*it)[1], params = (*it)[2];
+        std::vector<std::string> types;
+        size_t pos = 0;
+        while (pos < params.size()) {
+            size_t comma = params.find(',', pos);
+            if (comma == std::string::npos) comma = params.size();
+            std::string p = params.substr(pos, comma - pos);
+            pos = comma + 1;
+            // drop the parameter name (the last identifier)
+            size_t e = p.find_last_not_of(" \t\n");
+            if (e == std::string::npos) continue;
+            size_t b = e;
+            while (b > 0 && (std::isalnum((unsigned char)p[b - 1]) || p[b - 1] == '_')) b--;
+            std::string type = p.substr(0, b);
+            type = std::regex_replace(type, std::regex("__restrict__"), "");
+            types.push_back(type);
+        }
+        out += "extern \"C\" void " + name + "__emu(void** args)\n{\n    " + name + "(";
+        for (size_t i = 0; i < types.size(); i++)
+            out += (i ? ", " : "") + std::string("*(") + types[i] + "*)args[" + std::to_string(i) + "]";
+        out += ");\n}\n";
+    }
+    return out;
+}
+
+}  // namespace
+
 extern "C" {
 
 const char* ng_last_error(void) { return ng::g_err; }
 int ng_init(int device) { return ng::gemm_static_scratch_setup(device); }
+
+int ng_device_count(int* count) { *count = 1; return 0; }
+int ng_device_attr(int attr, int* value)
+{
+    switch (attr) {
+    case 0: *value = emu::g_cus; break;
+    case 1: *value = 160 * 1024; break;
+    case 2: *value = 64; break;
+    case 3: *value = 2400000; break;
+    case 4: *value = 2000000; break;
+    case 5: *value = 4 << 20; break;
+    default: return ng::fail(-5, "unknown device attribute %d", attr);
+    }
+    return 0;
+}
+int ng_device_name(char* buf, size_t cap) { snprintf(buf, cap, "lane-level CPU emulation (gfx950 kernels)"); return 0; }
+int ng_malloc(void** ptr, size_t bytes) { *ptr = emu_alloc(bytes); return *ptr ? 0 : ng::fail(-6, "out of memory"); }
+int ng_free(void* ptr) { emu_free(ptr); return 0; }
+int ng_mem_info(size_t* free_bytes, size_t* total_bytes) { *free_bytes = *total_bytes = (size_t)8 << 30; return 0; }
+int ng_memcpy_h2d(void* dst, const void* src, size_t bytes, void*) { std::memcpy(dst, src, bytes); return 0; }
+int ng_memcpy_d2h(void* dst, const void* src, size_t bytes, void*) { std::memcpy(dst, src, bytes); return 0; }
+int ng_memcpy_d2d(void* dst, const void* src, size_t bytes, void*) { std::memmove(dst, src, bytes); return 0; }
+int ng_memset8(void* dst, unsigned value, size_t count, void*) { std::memset(dst, (int)(value & 0xFF), count); return 0; }
+int ng_memset16(void* dst, unsigned value, size_t count, void*)
+{
+    unsigned short* p = (unsigned short*)dst;
+    for (size_t i = 0; i < count; i++) p[i] = (unsigned short)value;
+    return 0;
+}
+int ng_memset32(void* dst, unsigned value, size_t count, void*)
+{
+    unsigned* p = (unsigned*)dst;
+    for (size_t i = 0; i < count; i++) p[i] = value;
+    return 0;
+}
+int ng_stream_create(void** stream) { *stream = nullptr; return 0; }
+int ng_stream_sync(void*) { return 0; }
+int ng_stream_destroy(void*) { return 0; }
+int ng_event_create(void** event) { *event = (void*)1; return 0; }
+int ng_event_record(void*, void*) { return 0; }
+int ng_event_sync(void*) { return 0; }
+int ng_event_elapsed_ms(float* ms, void*, void*) { *ms = 1.0f; return 0; }
+int ng_event_destroy(void*) { return 0; }
+
+int ng_rtc_compile(const char* source, const char* name, const char** /*options*/, int /*n_options*/,
+                   void** module, char* log, size_t log_cap)
+{
+    *module = nullptr;
+    if (log && log_cap) log[0] = 0;
+    char tmpl[] = "/tmp/ng_emu_rtc_XXXXXX";
+    if (!mkdtemp(tmpl)) return ng::fail(-10, "mkdtemp failed");
+    const std::string dir(tmpl), cpp = dir + "/k.cpp", so = dir + "/k.so", err = dir + "/err.txt";
+    {
+        std::string text = std::string("#include <hip/hip_runtime.h>\n") + source + "\n" + trampolines(source);
+        FILE* f = fopen(cpp.c_str(), "w");
+        if (!f) return ng::fail(-10, "cannot write %s", cpp.c_str());
+        fwrite(text.data(), 1, text.size(), f);
+        fclose(f);
+    }
+    const std::string cmd = "/opt/rocm/llvm/bin/clang++ -std=c++17 -O1 -fPIC -shared -ffp-contract=off -I " + shim_dir() +
+                            " -Wno-psabi -Wno-unused-value -Wno-ignored-attributes -Wno-macro-redefined -x c++ " + cpp + " -x none " + this_library() +
+                            " -o " + so +
+                            " 2> " + err;
+    const int rc = system(cmd.c_str());
+    if (rc != 0) {
+        std::string msg;
+        if (FILE* f = fopen(err.c_str(), "r")) { char buf[2048]; size_t n = fread(buf, 1, sizeof(buf) - 1, f); buf[n] = 0; msg = buf; fclose(f); }
+        if (log && log_cap) { strncpy(log, msg.c_str(), log_cap - 1); log[log_cap - 1] = 0; }
+        return ng::fail(-11, "host compile of %s failed:\n%.700s", name, msg.c_str());
+    }
+    // the module finds emu::* and the other runtime symbols in this library (already loaded, global)
+    void* h = dlopen(so.c_str(), RTLD_NOW | RTLD_LOCAL);
+    if (!h) return ng::fail(-11, "dlopen(%s): %s", so.c_str(), dlerror());
+    *module = new EmuModule{h, dir};
+    return 0;
+}
+
+int ng_module_get_function(void** function, void* module, const char* name)
+{
+    EmuModule* m = (EmuModule*)module;
+    void* f = dlsym(m->handle, (std::string(name) + "__emu").c_str());
+    if (!f) return ng::fail(-12, "kernel %s not found in the emulated module", name);
+    *function = f;
+    return 0;
+}
+
+int ng_module_unload(void* module)
+{
+    EmuModule* m = (EmuModule*)module;
+    if (m) { dlclose(m->handle); delete m; }
+    return 0;
+}
+
+int ng_launch(void* function, const unsigned grid[3], const unsigned block[3], unsigned /*shared_bytes*/, void* /*stream*/,
+              void** args)
+{
+    if (!function) return ng::fail(-12, "ng_launch: null function");
+    if (grid[0] == 0 || grid[1] == 0 || grid[2] == 0) return 0;
+    if ((size_t)block[0] * block[1] * block[2] > 1024) return ng::fail(-13, "ng_launch: block too large");
+    void (*tramp)(void**) = (void (*)(void**))function;
+    emu::launch(dim3(grid[0], grid[1], grid[2]), dim3(block[0], block[1], block[2]), [=]() { tramp(args); });
+    return 0;
+}
+
 
 // controls of the emulation
 void emu_set_cus(int cus) { emu::g_cus = cus; }

@@ -18,6 +18,10 @@
 #include <cstdlib>
 #include <cstring>
 #include <functional>
+#include <math.h>
+using std::isfinite;
+using std::isinf;
+using std::isnan;
 
 #define __global__
 #define __device__
@@ -96,6 +100,10 @@ NG_EMU_MINMAX(long long) NG_EMU_MINMAX(unsigned long long) NG_EMU_MINMAX(float) 
 inline unsigned __float_as_uint(float f) { unsigned u; std::memcpy(&u, &f, 4); return u; }
 inline float __uint_as_float(unsigned u) { float f; std::memcpy(&f, &u, 4); return f; }
 inline float __uint2float_rn(unsigned u) { return (float)u; }
+inline float __builtin_amdgcn_rcpf(float x) { return 1.0f / x; }
+inline float __builtin_amdgcn_sqrtf(float x) { return std::sqrt(x); }
+inline int __shfl_xor(int v, int mask, int width);
+inline float __shfl_xor(float v, int mask, int width);
 
 // ---- scheduling hints and counters that need no emulation -------------------------------
 inline void __builtin_amdgcn_sched_barrier(int) {}
@@ -118,6 +126,15 @@ inline int __builtin_amdgcn_readlane(int v, int src_lane)
     emu::wave_exchange_sync();
     int r;
     std::memcpy(&r, slots + 64 * (src_lane & 63), 4);
+    return r;
+}
+inline int __shfl_xor(int v, int mask, int /*width*/)
+{
+    char* slots = emu::wave_exchange_begin();
+    std::memcpy(slots + 64 * emu::cur->lane, &v, 4);
+    emu::wave_exchange_sync();
+    int r;
+    std::memcpy(&r, slots + 64 * ((emu::cur->lane ^ mask) & 63), 4);
     return r;
 }
 inline float __shfl_xor(float v, int mask, int /*width*/)
