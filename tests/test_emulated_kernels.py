@@ -8,6 +8,7 @@ That checks index arithmetic, tile layouts, barriers and wait counts without a G
 numpy oracle as the GPU parity tests.  It is test infrastructure: the product never loads this library,
 and the results say nothing about speed."""
 import os
+import subprocess
 import sys
 
 import numpy as np
@@ -124,3 +125,19 @@ def test_emulated_pooling(emu, case):
             E = rng.uniform(-1, 1, O.shape).astype(np.float16)
             assert_fp16_within_ulp(emu.pool(op, I, JTRS, pad, strd, E=E), orc.ref_pool_bprop(I, E, name, JTRS, pad, strd),
                                    1.0, name + " bprop", 1e-6)
+
+
+CANDIDATES = [("fc", {"NG_FC_CFG": "1"}), ("fc", {"NG_FC_CFG": "2"}), ("fc", {"NG_FC_CFG": "3"}),
+              ("nt", {"NG_NT_STREAM": "1"}), ("nt", {"NG_NT_STREAM": "2"}), ("rows", {"NG_CONV_ROWS": "1"})]
+
+
+@pytest.mark.parametrize("what,switch", CANDIDATES)
+def test_emulated_candidate_kernels(emu, what, switch):
+    """kernels that wait behind environment switches for their first measurement on a device
+    (tests/emu/candidates.py): split k-steps inside a workgroup, the streamed outer-product GEMM,
+    the first-layer forward with decoded taps"""
+    env = dict(os.environ)
+    env.update(switch)
+    done = subprocess.run([sys.executable, os.path.join(os.path.dirname(os.path.abspath(__file__)), "emu", "candidates.py"), what],
+                          env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=900)
+    assert done.returncode == 0 and b"ok " + what.encode() in done.stdout, done.stdout.decode("utf-8", "replace")[-2000:]
