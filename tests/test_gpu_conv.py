@@ -304,6 +304,14 @@ def _sampled_layer_check(ng, layer, seed, gen, npix=256, nrows=6, in_dtype=np.fl
     rows = np.unique(np.concatenate([rng.integers(0, crst, nrows), [0, crst - 1]]))
     refu = orc.ref_conv_update_rows(If, E, layer.dimF, rows, layer.padding, layer.strides)
     assert_fp32_close(U[rows], refu, 1e-5, "update %s" % layer)
+    # the same gradient stored as fp16 (nervanagpu/nervanagpu.py:695-698, 723-724: fp32 accumulation, one
+    # rounding), at the configured shape: one unit in the last place of the fp32-accumulated value plus
+    # the accumulation slack of the sums over the absolute operands
+    dUh = ng.empty(layer.dimF, dtype=np.float16)
+    ng.update_conv(layer, dI, dE, dUh)
+    Uh = dUh.get().reshape(crst, layer.K)
+    absu = orc.ref_conv_update_rows(np.abs(If), np.abs(E.astype(np.float32)), layer.dimF, rows, layer.padding, layer.strides)
+    assert_fp16_within_ulp(Uh[rows], refu, 1.0, "update (fp16 out) %s" % layer, acc_atol(absu))
 
 
 def _alexnet_data(rng, layer):
