@@ -207,6 +207,9 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
             case 3: return launch_layout<_Float16, 128, 128, 128, 2, 1, true, 2, 4>(g, sr_bits);
             case 4: return launch_layout<_Float16, 64, 128, 64, 2, 1, true, 4, 2>(g, sr_bits);
             case 6: return launch_layout<_Float16, 128, 128, 64, 2, 2, true, 4, 2>(g, sr_bits);
+            case 7:   // few rows (m <= 2048): 32-row tiles, four wavefronts splitting a 128-deep tile
+                if (!g.trans_a && !g.trans_b) return launch_gemm<_Float16, 32, 128, 128, 1, 1, KC, MC, true, 3, 4>(g, sr_bits);
+                return launch_layout<_Float16, 64, 128, 64, 2, 1, true, 4, 2>(g, sr_bits);
             default: break;
             }
         }
@@ -271,7 +274,7 @@ size_t ng_gemm_workspace_bytes(int dtype, int trans_a, int trans_b, int m, int n
             splits = std::max(splits, choose_splits(ceil_div(m, bm) * ceil_div(n, bn) * batch_grid, total_k, 0, 0));
     // the minibatch-wide kernels (64-deep tiles or deeper) run one workgroup per CU
     if (dtype == NG_F16 && n <= 128)
-        for (int bm : {64, 128}) splits = std::max(splits, one_per_cu_splits(ceil_div(m, bm) * batch_grid, total_k, 0, 0));
+        for (int bm : {32, 64, 128}) splits = std::max(splits, one_per_cu_splits(ceil_div(m, bm) * batch_grid, total_k, 0, 0));
     if (splits <= 1) return 0;
     return (size_t)splits * batch_grid * m * n * sizeof(float);
 }
