@@ -234,7 +234,8 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
         }
     }
     if constexpr (!BLOCKED && std::is_same<TIN, _Float16>::value) {
-        // EXPERIMENT knob (to be removed): NG_CONV_ROWS=1 enables the filter-row streaming kernel
+        // A candidate that has passed the CPU emulation but has not been measured on a device yet: off unless
+        // NG_CONV_ROWS=1 (read once per process); it becomes the default, or goes, with its first measurement
         static const int tap_rows_on = getenv("NG_CONV_ROWS") ? atoi(getenv("NG_CONV_ROWS")) : 0;
         if (tap_rows_on) {
             // the kernel is compiled for the tile counts of the usual first layers: 7x7 on three

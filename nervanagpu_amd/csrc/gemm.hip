@@ -170,7 +170,8 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
     const int cus = device_cu_count();
     const int k_tiles = ceil_div(g.k, 64) * g.batch_loops;
     {
-        // EXPERIMENT knob (to be removed): NG_NT_STREAM=1 enables the streamed "nt" kernel
+        // A candidate that has passed the CPU emulation but has not been measured on a device yet: off unless
+        // NG_NT_STREAM is set (1: four ring stages, one workgroup per CU; 2: two stages, two per CU)
         static const int nt_stream = getenv("NG_NT_STREAM") ? atoi(getenv("NG_NT_STREAM")) : 0;
         if (nt_stream && nt_streams(g, sr_bits)) {
             if (g.k <= 64) return sr_bits ? launch_nt_stream<2, true>(g, sr_bits) : launch_nt_stream<2, false>(g, sr_bits);
@@ -198,7 +199,8 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
         return launch_layout<_Float16, 128, 128, 64, 2, 2, true>(g, sr_bits);
     }
     if (g.n <= 128) {
-        // EXPERIMENT knob (to be removed): NG_FC_CFG picks the minibatch-wide kernel
+        // Candidates that have passed the CPU emulation but have not been measured on a device yet: NG_FC_CFG
+        // (read once per process) picks one; unset, the measured 64x128x64 tile on 2x2 wavefronts runs
         static const int fc_cfg = getenv("NG_FC_CFG") ? atoi(getenv("NG_FC_CFG")) : 0;
         if (g.n > 64 && g.batch_grid == 1 && k_tiles >= 8) {
             switch (fc_cfg) {
