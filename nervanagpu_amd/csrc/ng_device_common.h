@@ -91,18 +91,18 @@ NG_DEV unsigned short ng_sr_f16(float v, unsigned bits, unsigned r)
     return ng_f32_to_f16_rz(__uint_as_float((u & 0x80000000u) | m2));
 }
 
-// The same rounding when all 10 mantissa bits of fp16 are kept, in fewer
-// operations.  The truncating convert drops exactly the bits the mask would
-// clear; bounding the sum by max(mag, largest finite fp32) keeps the increment
-// from carrying a finite value into the infinity pattern (the convert then
-// saturates at 65504 as the clamp did) and leaves infinities and NaNs as they
-// are.  Returns the fp32 value whose truncating convert is the result.
+// The same rounding when all 10 mantissa bits of fp16 are kept, in three
+// operations (add, compare, select).  The truncating convert drops exactly the
+// bits the mask would clear, and the sign bit sits above every carry, so the
+// increment is added to the signed pattern as it is.  Magnitudes within 2^13
+// patterns of the largest finite fp32 could carry into the infinity pattern:
+// they, infinities and NaNs are passed on unchanged (the convert saturates the
+// former at 65504, as the clamp did, whatever was added).  Returns the fp32
+// value whose truncating convert is the result.
 NG_DEV float ng_sr10_bump(float v, unsigned r13)
 {
-    const unsigned u   = __float_as_uint(v);
-    const unsigned mag = u & 0x7FFFFFFFu;
-    const unsigned m2  = min(mag + r13, max(mag, 0x7F7FFFFFu));
-    return __uint_as_float((u & 0x80000000u) | m2);
+    const float bumped = __uint_as_float(__float_as_uint(v) + r13);
+    return (__builtin_fabsf(v) < __uint_as_float(0x7F7FE000u)) ? bumped : v;
 }
 
 // Two neighbouring elements sharing the draw h (even element: its high half,
