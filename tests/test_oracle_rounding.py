@@ -143,17 +143,20 @@ def test_fast_ew_dims():
 
 def test_sr10_short_form_is_the_same_function():
     """The device rounds at the default 10 bits with a shorter expression
-    (ng_sr10_bump in csrc/ng_device_common.h): no mask, and the sum bounded by
-    max(magnitude, largest finite fp32) instead of clamp + infinity test.  It
-    must be the oracle's function bit for bit, NaN payloads included."""
+    (ng_sr10_bump in csrc/ng_device_common.h): no mask, the increment added to
+    the signed pattern as it is, and values whose magnitude lies within 2^13
+    patterns of the largest finite fp32 (or beyond: infinities, NaNs) passed on
+    unchanged instead of clamp + infinity test.  It must be the oracle's
+    function bit for bit, NaN payloads included."""
     U = np.uint32
 
     def short_form(x, r):
-        u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
-        mag = u & U(0x7FFFFFFF)
-        with np.errstate(over="ignore"):
-            t = np.minimum(mag + (r >> U(19)), np.maximum(mag, U(0x7F7FFFFF)))
-        return rn.f32_to_f16_rz(((u & U(0x80000000)) | t).astype(np.uint32).view(np.float32))
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        u = x.view(np.uint32)
+        with np.errstate(over="ignore", invalid="ignore"):
+            bumped = (u + (r >> U(19))).astype(np.uint32)
+            keep = np.abs(x) < np.array([0x7F7FE000], dtype=np.uint32).view(np.float32)[0]
+        return rn.f32_to_f16_rz(np.where(keep, bumped, u).astype(np.uint32).view(np.float32))
 
     rng = np.random.default_rng(3)
     for case in range(4):
