@@ -366,6 +366,35 @@ def test_stochastic_rounding_bit_exact(ng):
     assert np.all(np.abs(got - ref) <= 2.0 ** -7 * np.abs(ref) * 1.01 + 1e-5)   # within one unit at 7 bits
 
 
+def test_batched_dot_stochastic_rounding_bit_exact():
+    """stochastic stores through batched_dot: one product per batch entry (the random stream is indexed
+    by the flat position in the (batch, m, n) result) and the sum over the batch into a 2-D result, both
+    bit for bit against the numpy restatement fed the same stream.  Dyadic operands: every fp32 sum is
+    exact, so the value before rounding is known without ambiguity."""
+    from nervanagpu_amd import NervanaGPU
+    ngs = NervanaGPU(stochastic_round=10, seed=77)
+    rng = np.random.default_rng(21)
+    X, nOut, nIn, N = 6, 96, 72, 32
+    W = _dyadic(rng, (nOut, nIn), 32)
+    I = _dyadic(rng, (X, nIn, N), 32)
+    E = _dyadic(rng, (X, nOut, N), 32)
+    dW, dI, dE = ngs.array(W), ngs.array(I), ngs.array(E)
+    dO = ngs.empty((X, nOut, N))
+    ngs.batched_dot(dW, dI, dO, relu=True)
+    pre = np.maximum(orc.ref_batched_dot(W, I, acc_dtype=np.float32), 0)
+    assert np.array_equal(pre.astype(np.float64), np.maximum(np.einsum("oi,xin->xon", W.astype(np.float64), I.astype(np.float64)), 0))
+    r = orc.rand_sr16(77, ngs.rng_counter, np.arange(pre.size, dtype=np.uint32)).reshape(pre.shape)
+    got = dO.get()
+    assert np.array_equal(got.view(np.uint16), orc.round_stochastic_fp16(pre, 10, r).view(np.uint16))
+    assert not np.array_equal(got.view(np.uint16), pre.astype(np.float16).view(np.uint16))
+    dU = ngs.empty((nOut, nIn))
+    ngs.batched_dot(dE, dI.T, dU)
+    pre = orc.ref_batched_dot(E, np.transpose(I, (0, 2, 1)), out_3d=False, acc_dtype=np.float32)
+    assert np.array_equal(pre.astype(np.float64), np.einsum("xon,xin->oi", E.astype(np.float64), I.astype(np.float64)))
+    r = orc.rand_sr16(77, ngs.rng_counter, np.arange(pre.size, dtype=np.uint32)).reshape(pre.shape)
+    assert np.array_equal(dU.get().view(np.uint16), orc.round_stochastic_fp16(pre, 10, r).view(np.uint16))
+
+
 def _dyadic(rng, shape, step=16):
     """multiples of 1/step in [-1, 1]: products are multiples of 1/step^2, and
     sums of up to 2^14 of them are exact in fp32 in any order"""
