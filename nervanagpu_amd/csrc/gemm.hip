@@ -308,7 +308,8 @@ int ng_gemm(int dtype, int trans_a, int trans_b, int m, int n, int k,
 static __device__ __align__(256) unsigned char scratch[NG_GEMM_STATIC_SCRATCH_BYTES];
 
 static constexpr int MAX_DEVICES = 64;
-static void* g_scratch_ptr[MAX_DEVICES];
+// written once per device under the mutex, read by every call without it
+static std::atomic<void*> g_scratch_ptr[MAX_DEVICES];
 static std::mutex g_scratch_mutex;
 // The nervana_* entry points also put their partial sums into the array.  Their
 // callers may use several streams, so the last call that used it leaves an event
@@ -323,7 +324,7 @@ int gemm_static_scratch_setup(int device)
 {
     if (device < 0 || device >= MAX_DEVICES) return fail(-30, "device index %d out of range", device);
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    if (g_scratch_ptr[device]) return 0;
+    if (g_scratch_ptr[device].load(std::memory_order_acquire)) return 0;
     void* ptr = nullptr;
     hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
@@ -331,7 +332,7 @@ int gemm_static_scratch_setup(int device)
     e = hipEventCreateWithFlags(&g_scratch_order[device].done, hipEventDisableTiming);
     if (e != hipSuccess) return hip_fail(e, "hipEventCreateWithFlags(scratch order)");
     g_scratch_order[device].used = false;
-    g_scratch_ptr[device] = ptr;
+    g_scratch_ptr[device].store(ptr, std::memory_order_release);
     return 0;
 }
 
@@ -350,8 +351,8 @@ int ng_gemm_noalloc(int dtype, int trans_a, int trans_b, int m, int n, int k,
 {
     int dev = -1;
     NG_HIP(hipGetDevice(&dev));
-    if (dev < 0 || dev >= MAX_DEVICES || !g_scratch_ptr[dev])
-        return fail(-32, "ng_gemm_noalloc: ng_init has not been called for device %d", dev);
+    void* const arena = (dev >= 0 && dev < MAX_DEVICES) ? g_scratch_ptr[dev].load(std::memory_order_acquire) : nullptr;
+    if (!arena) return fail(-32, "ng_gemm_noalloc: ng_init has not been called for device %d", dev);
     if (m < 0 || n < 0 || k < 0 || batch_grid < 1 || batch_loops < 1)
         return fail(-22, "ng_gemm_noalloc: bad extent");
     const size_t need = ng_gemm_workspace_bytes(dtype, trans_a, trans_b, m, n, k, batch_grid, batch_loops);
@@ -362,7 +363,7 @@ int ng_gemm_noalloc(int dtype, int trans_a, int trans_b, int m, int n, int k,
     // reads them, so nothing in the array has to start at zero
     return ng_gemm(dtype, trans_a, trans_b, m, n, k, A, lda, B, ldb, C, ldc, alpha, beta, flags, seed, rng_stream,
                    batch_grid, ldaz, ldbz, ldcz, batch_loops,
-                   need ? g_scratch_ptr[dev] : nullptr, need, stream);
+                   need ? arena : nullptr, need, stream);
 }
 
 // ---- GEMM-only C interface (kernels/C_interface/nervana_c_api.h) -----------
@@ -393,8 +394,11 @@ static bool c_gemm(int dtype, void* A, void* B, void* C, bool a_t, bool b_t, int
     // static array, so this entry runs the same schedule as NervanaGPU.dot.
     int dev = -1;
     const size_t need = (m > 0 && n > 0 && k > 0) ? ng_gemm_workspace_bytes(dtype, a_t, b_t, m, n, k, 1, 1) : 0;
-    const bool sliced = need > 0 && need <= (size_t)NG_GEMM_STATIC_SCRATCH_BYTES &&
-                        hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < MAX_DEVICES && g_scratch_ptr[dev];
+    void* arena = nullptr;
+    if (need > 0 && need <= (size_t)NG_GEMM_STATIC_SCRATCH_BYTES && hipGetDevice(&dev) == hipSuccess && dev >= 0 &&
+        dev < MAX_DEVICES)
+        arena = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    const bool sliced = arena != nullptr;
     int rc;
     if (sliced) {
         std::lock_guard<std::mutex> lock(g_scratch_mutex);
@@ -403,7 +407,7 @@ static bool c_gemm(int dtype, void* A, void* B, void* C, bool a_t, bool b_t, int
         if (ord.used && ord.last != (hipStream_t)stream) e = hipStreamWaitEvent((hipStream_t)stream, ord.done, 0);
         rc = (e != hipSuccess) ? hip_fail(e, "hipStreamWaitEvent(scratch order)")
                                : ng_gemm(dtype, a_t, b_t, m, n, k, A, lda, B, ldb, C, ldc, alpha, beta, flags,
-                                         0u, rng_stream, 1, 0, 0, 0, 1, g_scratch_ptr[dev], need, stream);
+                                         0u, rng_stream, 1, 0, 0, 0, 1, arena, need, stream);
         if (rc == 0) {
             e = hipEventRecord(ord.done, (hipStream_t)stream);
             if (e != hipSuccess) rc = hip_fail(e, "hipEventRecord(scratch order)");
