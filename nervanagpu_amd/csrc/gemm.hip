@@ -56,7 +56,8 @@ static int one_per_cu_splits(int out_tiles, int total_k_tiles, size_t slice_byte
     return std::max(splits, 1);
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, bool VEC, int NSTAGE = 2, int WK = 1>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int LA, int LB, bool VEC, int NSTAGE = 2, int WK = 1,
+          bool ONE_PER_CU = (WK > 1)>
 static int launch_gemm(const GemmArgs& g, unsigned sr_bits)
 {
     CoreShape s;
@@ -68,7 +69,7 @@ static int launch_gemm(const GemmArgs& g, unsigned sr_bits)
     const int zcount = g.batch_grid;
     const int out_tiles = s.tiles_m * s.tiles_n * zcount;
     const size_t slice_bytes = (size_t)zcount * g.m * g.n * sizeof(float);
-    if (WK > 1) s.splits = g.ws ? one_per_cu_splits(out_tiles, s.passes * s.k_tiles, slice_bytes, g.ws_bytes) : 1;
+    if (ONE_PER_CU) s.splits = g.ws ? one_per_cu_splits(out_tiles, s.passes * s.k_tiles, slice_bytes, g.ws_bytes) : 1;
     else        s.splits = g.ws ? choose_splits(out_tiles, s.passes * s.k_tiles, slice_bytes, g.ws_bytes) : 1;
 
     DenseLoader<T, LA, VEC> al{(const T*)g.A, g.ldaz, g.lda, g.m, g.k};
@@ -91,12 +92,12 @@ static int launch_gemm(const GemmArgs& g, unsigned sr_bits)
     return 0;
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, bool VEC, int NSTAGE = 2, int WK = 1>
+template <typename T, int BM, int BN, int BK, int WM, int WN, bool VEC, int NSTAGE = 2, int WK = 1, bool ONE_PER_CU = (WK > 1)>
 static int launch_layout(const GemmArgs& g, unsigned sr_bits)
 {
-    if (!g.trans_a && !g.trans_b) return launch_gemm<T, BM, BN, BK, WM, WN, KC, MC, VEC, NSTAGE, WK>(g, sr_bits);
-    if (!g.trans_a && g.trans_b)  return launch_gemm<T, BM, BN, BK, WM, WN, KC, KC, VEC, NSTAGE, WK>(g, sr_bits);
-    return launch_gemm<T, BM, BN, BK, WM, WN, MC, MC, VEC, NSTAGE, WK>(g, sr_bits);
+    if (!g.trans_a && !g.trans_b) return launch_gemm<T, BM, BN, BK, WM, WN, KC, MC, VEC, NSTAGE, WK, ONE_PER_CU>(g, sr_bits);
+    if (!g.trans_a && g.trans_b)  return launch_gemm<T, BM, BN, BK, WM, WN, KC, KC, VEC, NSTAGE, WK, ONE_PER_CU>(g, sr_bits);
+    return launch_gemm<T, BM, BN, BK, WM, WN, MC, MC, VEC, NSTAGE, WK, ONE_PER_CU>(g, sr_bits);
 }
 
 // B operand of the streaming kernel for a dense "nt" product: column c of the
@@ -212,6 +213,9 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
             case 7:   // few rows (m <= 2048): 32-row tiles, four wavefronts splitting a 128-deep tile
                 if (!g.trans_a && !g.trans_b) return launch_gemm<_Float16, 32, 128, 128, 1, 1, KC, MC, true, 3, 4>(g, sr_bits);
                 return launch_layout<_Float16, 64, 128, 64, 2, 1, true, 4, 2>(g, sr_bits);
+            // the same rows without the in-workgroup split: a whole CU of LDS as stages of the weight stream
+            case 8: return launch_layout<_Float16, 128, 128, 32, 2, 2, true, 8, 1, true>(g, sr_bits);
+            case 9: return launch_layout<_Float16, 128, 128, 64, 2, 2, true, 4, 1, true>(g, sr_bits);
             default: break;
             }
         }
