@@ -213,6 +213,9 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
             case 7:   // few rows (m <= 2048): 32-row tiles, four wavefronts splitting a 128-deep tile
                 if (!g.trans_a && !g.trans_b) return launch_gemm<_Float16, 32, 128, 128, 1, 1, KC, MC, true, 3, 4>(g, sr_bits);
                 return launch_layout<_Float16, 64, 128, 64, 2, 1, true, 4, 2>(g, sr_bits);
+            case 10:  // as 7 with a fourth stage: the four tiles of a 512-deep slice are all requested at once
+                if (!g.trans_a && !g.trans_b) return launch_gemm<_Float16, 32, 128, 128, 1, 1, KC, MC, true, 4, 4>(g, sr_bits);
+                return launch_layout<_Float16, 64, 128, 64, 2, 1, true, 4, 2>(g, sr_bits);
             // the same rows without the in-workgroup split: a whole CU of LDS as stages of the weight stream
             case 8: return launch_layout<_Float16, 128, 128, 32, 2, 2, true, 8, 1, true>(g, sr_bits);
             case 9: return launch_layout<_Float16, 128, 128, 64, 2, 2, true, 4, 1, true>(g, sr_bits);
