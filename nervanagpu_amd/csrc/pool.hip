@@ -19,6 +19,7 @@
 #include "ng_device_common.h"
 
 #include <algorithm>
+#include <cstdlib>
 
 namespace ng {
 
@@ -98,6 +99,10 @@ struct PoolGeom {
     // that hold at least one input element
     int use_cells, cells_h, cells_w, cell_remap;
     FastDiv div_ch, div_cw;
+    // backward by cells on maps of fewer workgroups: whole feature maps per XCD
+    // (see xcd_map_block); div_cell_blocks divides by the workgroups of one map
+    int cell_map_xcd;
+    FastDiv div_cell_blocks;
     // max pooling backward with the rectifier derivative of the layer below
     // folded in: a window whose maximum is not positive passes nothing on
     int relu_mask;
@@ -119,6 +124,21 @@ enum { NO_SLOT = 255 };
 __device__ __forceinline__ unsigned xcd_block_index(int remap)
 {
     return remap ? (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3) : blockIdx.x;
+}
+
+// Whole feature maps per XCD, for maps too small to cut into eighths: workgroups
+// are handed to the 8 XCDs in turn in launch order (x fastest), so workgroup
+// L = y * gridDim.x + x runs on XCD L % 8.  That XCD works through the maps
+// xcd, xcd + 8, xcd + 16, ... one after the other: the windows two neighbouring
+// rows of cells share are then fetched into one L2 once instead of into two.
+// Needs gridDim.y (the feature maps) to be a multiple of 8.
+__device__ __forceinline__ void xcd_map_block(const FastDiv& blocks_per_map, unsigned& block, unsigned& map)
+{
+    const unsigned linear = blockIdx.y * gridDim.x + blockIdx.x;
+    const unsigned turn = linear >> 3;
+    const unsigned round = blocks_per_map.div(turn);
+    block = turn - round * gridDim.x;
+    map = round * 8u + (linear & 7u);
 }
 
 __device__ __forceinline__ bool split_inner(unsigned inner, unsigned limit, const FastDiv& dn, const FastDiv& d1,
@@ -444,14 +464,16 @@ void pool_bprop_cell_kernel(const T* __restrict__ E, const unsigned char* __rest
     constexpr int NW = (RS + STR - 1) / STR;
     typedef typename Pack<T, VEC>::raw_t raw_t;
     const unsigned per_map = (unsigned)(g.D * g.cells_h * g.cells_w * g.nvec);
-    const unsigned inner = xcd_block_index(g.cell_remap) * 256u + threadIdx.x;
+    unsigned block = xcd_block_index(g.cell_remap), map = blockIdx.y;
+    if (g.cell_map_xcd) xcd_map_block(g.div_cell_blocks, block, map);
+    const unsigned inner = block * 256u + threadIdx.x;
     int nv, cx, cy, z;
     if (!split_inner(inner, per_map, g.div_nvec, g.div_cw, g.div_ch, g.nvec, g.cells_w, g.cells_h, nv, cx, cy, z)) return;
     // one feature map holds fewer than 2^31 elements: 32-bit offsets inside it
-    const long out_map = (long)blockIdx.y * g.M * g.P * g.Q * g.N;
+    const long out_map = (long)map * g.M * g.P * g.Q * g.N;
     const T* Em = E + out_map;
     const unsigned char* am = arg + (OP == OP_MAX ? out_map : 0);
-    T* Bm = B + (long)blockIdx.y * g.D * g.H * g.W * g.N;
+    T* Bm = B + (long)map * g.D * g.H * g.W * g.N;
 
     raw_t eraw[NW * NW];
     unsigned words[NW * NW][2];
@@ -630,6 +652,14 @@ static PoolGeom make_geom(const ng_pool_params& p, int vec, size_t elem_bytes)
     g.cell_remap = (!disjoint && (long)p.D * g.cells_h * g.cells_w * g.nvec >= 64 * 256) ? 1 : 0;
     g.div_ch = FastDiv::make((unsigned)g.cells_h);
     g.div_cw = FastDiv::make((unsigned)g.cells_w);
+    // smaller maps: whole maps per XCD when the maps divide over the 8 XCDs (the
+    // 56x56 maps of 128 images are 49 workgroups: without it consecutive
+    // workgroups, i.e. neighbouring rows of cells, sit on different XCDs and the
+    // errors and argmax bytes are fetched twice: 152 MB for 72 MB)
+    const long cell_blocks = ((long)p.D * g.cells_h * g.cells_w * g.nvec + 255) / 256;
+    static const bool map_xcd_off = getenv("NG_POOL_MAP_XCD") && atoi(getenv("NG_POOL_MAP_XCD")) == 0;
+    g.cell_map_xcd = (!disjoint && !g.cell_remap && p.C % 8 == 0 && cell_blocks >= 2 && !map_xcd_off) ? 1 : 0;
+    g.div_cell_blocks = FastDiv::make((unsigned)cell_blocks);
     return g;
 }
 

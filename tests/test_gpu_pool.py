@@ -25,6 +25,11 @@ CASES = [
     (8, 10, 1, 5, 5, 3, 1, 1, 1, (1, 0, 0, 0), (2, 1, 1, 1)),        # overlapping, padded windows over feature maps
     (8, 4, 7, 6, 6, 1, 3, 2, 2, (0, 1, 0, 0), (1, 2, 2, 2)),         # overlapping in depth only
     (8, 3, 1, 9, 8, 1, 1, 2, 2, (0, 0, 0, 0), (1, 1, 1, 1)),         # 2x2/1: overlapping, no compiled cell shape
+    # feature maps in multiples of 8 and several workgroups of cells per map: the backward kernel numbers its
+    # workgroups so that an XCD takes whole maps
+    (64, 16, 1, 13, 13, 1, 1, 3, 3, (0, 0, 0, 0), (1, 1, 2, 2)),     # 3x3/2, two workgroups per map
+    (32, 24, 1, 20, 18, 1, 1, 3, 3, (0, 0, 1, 1), (1, 1, 2, 2)),     # 3x3/2 padded, 24 maps
+    (32, 8, 1, 10, 9, 1, 1, 3, 3, (0, 0, 1, 1), (1, 1, 1, 1)),       # 3x3/1 padded
 ]
 
 
