@@ -103,6 +103,9 @@ struct PoolGeom {
     // (see xcd_map_block); div_cell_blocks divides by the workgroups of one map
     int cell_map_xcd;
     FastDiv div_cell_blocks;
+    // the same numbering for the forward kernels (instead of xcd_remap)
+    int fwd_map_xcd;
+    FastDiv div_fwd_blocks;
     // max pooling backward with the rectifier derivative of the layer below
     // folded in: a window whose maximum is not positive passes nothing on
     int relu_mask;
@@ -194,8 +197,10 @@ __global__ __launch_bounds__(256)
 void pool_fprop_kernel(const T* __restrict__ I, T* __restrict__ O, unsigned char* __restrict__ arg, PoolGeom g)
 {
     const unsigned per_map = (unsigned)(g.M * g.P * g.Q * g.nvec);
-    const unsigned inner = xcd_block_index(g.xcd_remap) * 256u + threadIdx.x;
-    const int k = blockIdx.y;
+    unsigned block = xcd_block_index(g.xcd_remap), map = blockIdx.y;
+    if (g.fwd_map_xcd) xcd_map_block(g.div_fwd_blocks, block, map);
+    const unsigned inner = block * 256u + threadIdx.x;
+    const int k = (int)map;
     int nv, q, p, m;
     if (!split_inner(inner, per_map, g.div_nvec, g.div_q, g.div_p, g.nvec, g.Q, g.P, nv, q, p, m)) return;
     const int c0 = k * g.str_j - g.pad_j, z0 = m * g.str_d - g.pad_d;
@@ -657,9 +662,15 @@ static PoolGeom make_geom(const ng_pool_params& p, int vec, size_t elem_bytes)
     // workgroups, i.e. neighbouring rows of cells, sit on different XCDs and the
     // errors and argmax bytes are fetched twice: 152 MB for 72 MB)
     const long cell_blocks = ((long)p.D * g.cells_h * g.cells_w * g.nvec + 255) / 256;
-    static const bool map_xcd_off = getenv("NG_POOL_MAP_XCD") && atoi(getenv("NG_POOL_MAP_XCD")) == 0;
-    g.cell_map_xcd = (!disjoint && !g.cell_remap && p.C % 8 == 0 && cell_blocks >= 2 && !map_xcd_off) ? 1 : 0;
+    // NG_POOL_MAP_XCD (read once): 0 = launch-order numbering as before; 2 = also the forward kernels of
+    // such maps (16 to 63 workgroups per map are cut into eighths today: a candidate, not measured yet)
+    static const int map_xcd = getenv("NG_POOL_MAP_XCD") ? atoi(getenv("NG_POOL_MAP_XCD")) : 1;
+    g.cell_map_xcd = (!disjoint && !g.cell_remap && p.C % 8 == 0 && cell_blocks >= 2 && map_xcd != 0) ? 1 : 0;
     g.div_cell_blocks = FastDiv::make((unsigned)cell_blocks);
+    const long fwd_blocks = ((long)p.M * p.P * p.Q * g.nvec + 255) / 256;
+    g.fwd_map_xcd = (map_xcd == 2 && !disjoint && p.K % 8 == 0 && fwd_blocks >= 2 && fwd_blocks < 64) ? 1 : 0;
+    if (g.fwd_map_xcd) g.xcd_remap = 0;
+    g.div_fwd_blocks = FastDiv::make((unsigned)fwd_blocks);
     return g;
 }
 
