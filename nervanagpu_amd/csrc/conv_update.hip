@@ -4,7 +4,9 @@
 // slices of the (pixel, n) range are added in a fixed order instead of with
 // fp32 atomics, so the result does not depend on execution order.
 #include "conv_plan.h"
+#include <cstdlib>
 #include "conv_update_ring.h"
+#include "conv_update_strip.h"
 
 namespace ng {
 
@@ -90,6 +92,52 @@ static int launch_update_ring(const ConvPlan& pl, const void* I, const void* E, 
     return 0;
 }
 
+// 3x3 filters, padding 1, unit strides, one image plane, 64 images, 33 to 64 channels and at most
+// 64 output maps: the strip kernel (conv_update_strip.h), all nine taps on one ring
+static bool update_walks_strips(const ConvPlan& pl)
+{
+    const ng_conv_params& p = pl.p;
+    return p.R == 3 && p.S == 3 && p.T == 1 && p.D == 1 && p.pad_d == 0 && p.pad_h == 1 && p.pad_w == 1 &&
+           p.str_d == 1 && p.str_h == 1 && p.str_w == 1 && p.N == 64 && p.C > 32 && p.C <= 64 && p.K <= 64 && p.K % 8 == 0 &&
+           p.P == p.H && p.Q == p.W && p.W >= 8 &&
+           (long)p.C * p.H * p.W * p.N * 2 < (1L << 31) && (long)p.K * p.P * p.Q * p.N * 2 < (1L << 31);
+}
+
+template <typename TOUT>
+static int launch_update_strip(const ConvPlan& pl, const void* I, const void* E, void* gradF, float alpha,
+                               void* ws, size_t ws_bytes, hipStream_t stream)
+{
+    constexpr int WT = 4, LEAD = 2;
+    const ng_conv_params& p = pl.p;
+    const int rows = pl.CRST, cols = p.K;
+    CoreShape s;
+    s.m = rows; s.n = cols;
+    s.tiles_m = 1; s.tiles_n = 1;
+    s.passes = 1;
+    const int strips = cdiv(p.W, WT);
+    const int steps = strips * (p.H + 2) * (WT + 2);
+    s.k_tiles = steps;
+    const size_t slice = (size_t)rows * cols * sizeof(float);
+    s.splits = ws ? conv_splits(1, steps, slice, ws_bytes, 1) : 1;
+    UpdateStripGeom g{(const _Float16*)I, (const _Float16*)E, p.C, p.K, p.H, p.W, strips, p.H * p.W * p.N,
+                      p.P * p.Q * p.N, steps, FastDiv::make((unsigned)(WT + 2)), FastDiv::make((unsigned)(p.H + 2))};
+    ScaleStoreEpilogue<TOUT> epi{(TOUT*)gradF, 0, p.K, rows, cols, alpha, 0.0f, 0u, 0u, 0u, 0u,
+                                 (((uintptr_t)gradF & 15) == 0) ? 1u : 0u};
+    const dim3 grid(grid_tiles(1, s.splits), grid_slices(1, s.splits), 1);
+    const dim3 block(768);
+    if (s.splits == 1) {
+        hipLaunchKernelGGL((conv_update_strip_kernel<WT, LEAD, ScaleStoreEpilogue<TOUT>>), grid, block, 0, stream, g, epi, s);
+        NG_CHECK_LAUNCH("conv update (strips)");
+        return 0;
+    }
+    PartialEpilogue pe{(float*)ws, rows, cols, 1, 1u};
+    hipLaunchKernelGGL((conv_update_strip_kernel<WT, LEAD, PartialEpilogue>), grid, block, 0, stream, g, pe, s);
+    NG_CHECK_LAUNCH("conv update (strips)");
+    launch_splitk_reduce<TOUT, ScaleStoreEpilogue<TOUT>>((const float*)ws, s.splits, 1, rows, cols, epi, stream);
+    NG_CHECK_LAUNCH("conv update reduce");
+    return 0;
+}
+
 template <typename TIN, typename TOUT>
 static int update_h(const ConvPlan& pl, const void* I, const void* E, void* gradF, float alpha,
                     void* ws, size_t ws_bytes, hipStream_t st)
@@ -97,6 +145,12 @@ static int update_h(const ConvPlan& pl, const void* I, const void* E, void* grad
     if (pl.p.N % 64 == 0) {
         // fp16 activations: tile shaped after the filter matrix (CRST x K)
         if constexpr (std::is_same<TIN, _Float16>::value) {
+            {
+                // A candidate that has passed the CPU emulation but has not been measured on a device yet:
+                // off unless NG_UPDATE_STRIPS=1 (read once per process)
+                static const int strips_on = getenv("NG_UPDATE_STRIPS") ? atoi(getenv("NG_UPDATE_STRIPS")) : 0;
+                if (strips_on && update_walks_strips(pl)) return launch_update_strip<TOUT>(pl, I, E, gradF, alpha, ws, ws_bytes, st);
+            }
             if (update_shares_taps(pl)) {
                 // all rows of a 64-channel 3x3 filter in one workgroup of twelve wavefronts (E is
                 // then requested once instead of once per 64 rows; VGG conv1.2 0.47 -> 0.38 ms),

@@ -385,13 +385,15 @@ template <class E, class = void> struct EpilogueBufferStore { static constexpr b
 template <class E> struct EpilogueBufferStore<E, std::enable_if_t<E::BUFFER_STORE>> { static constexpr bool value = true; };
 
 // ROW_TAPS > 1: the TM bands of a wavefront are ROW_TAPS interleaved row sets (band
-// I holds rows (mbase + (I / ROW_TAPS) * 32 + r) * ROW_TAPS + I % ROW_TAPS: the
-// horizontal taps of 32 filter rows of the weight gradient's ring kernel)
-template <int TM, int TN, int WTN, int EPITCH, int I, int ROW_TAPS = 1>
+// I holds rows (mbase + ((I / ROW_TAPS) * 32 + r) * ROW_STRIDE) * ROW_TAPS + I % ROW_TAPS:
+// the horizontal taps of 32 filter rows of the weight gradient's ring kernel; with
+// ROW_STRIDE 3 those rows are one vertical tap of 32 channels of a 3x3 filter)
+template <int TM, int TN, int WTN, int EPITCH, int I, int ROW_TAPS = 1, int ROW_STRIDE = 1>
 struct EpilogueBands {
     static __device__ __forceinline__ int row_of(int mbase, int r)
     {
-        return ROW_TAPS == 1 ? mbase + I * 32 + r : (mbase + (I / ROW_TAPS) * 32 + r) * ROW_TAPS + I % ROW_TAPS;
+        return ROW_TAPS == 1 ? mbase + I * 32 + r
+                             : (mbase + ((I / ROW_TAPS) * 32 + r) * ROW_STRIDE) * ROW_TAPS + I % ROW_TAPS;
     }
     template <class Epi>
     static __device__ __forceinline__ void run(float16_t (&acc)[TM][TN], char* stage, int lane,
@@ -441,7 +443,7 @@ struct EpilogueBands {
         }
         wave_lds_fence();
         if constexpr (I + 1 < TM)
-            EpilogueBands<TM, TN, WTN, EPITCH, I + 1, ROW_TAPS>::run(acc, stage, lane, mbase, nbase, z, split, epi);
+            EpilogueBands<TM, TN, WTN, EPITCH, I + 1, ROW_TAPS, ROW_STRIDE>::run(acc, stage, lane, mbase, nbase, z, split, epi);
     }
 };
 

@@ -5,8 +5,10 @@ device (the switches are read once per process, hence this separate script):
                        or that spend a whole CU of LDS on stages of the weight stream
     NG_NT_STREAM=1|2   outer-product GEMM: rows of A resident in registers, output columns streamed
     NG_CONV_ROWS=1     first-layer forward with large filters: taps decoded from the contraction row
+    NG_UPDATE_STRIPS=1 weight gradient of 3x3 filters with at most 64 channels and output maps: strips of four
+                       output columns, all nine taps on one ring of input pixels
 
-usage: python tests/emu/candidates.py fc|nt|rows   (with the switch set in the environment)
+usage: python tests/emu/candidates.py fc|nt|rows|strips   (with the switch set in the environment)
 Every case runs with loads landing at once and with loads landing as late as the wait counts allow."""
 import os
 import sys
@@ -78,6 +80,22 @@ def rows():
             assert_fp16_within_ulp(got, ref, 1.0, "rows %s" % ((N, C, K, DHW, TRS, late),), acc_atol(C * np.prod(TRS)))
 
 
+def strips():
+    rng = np.random.default_rng(4)
+    # (N, C, K, H, W): widths that are and are not multiples of the strip, fewer channels / maps than 64,
+    # one CU (a single slice walks every strip) and eight (slices start inside strips)
+    for (N, C, K, H, W, cus) in [(64, 64, 64, 6, 8, 8), (64, 64, 64, 9, 10, 1), (64, 40, 24, 5, 13, 8), (64, 64, 48, 12, 9, 3)]:
+        conv = emu.Conv(np.float16, N, C, K, (1, H, W), (1, 3, 3), (0, 1, 1), (1, 1, 1), cus=cus)
+        I = rng.uniform(-1, 1, conv.dimI).astype(np.float16)
+        E = rng.uniform(-1, 1, conv.dimO).astype(np.float16)
+        ref = orc.ref_conv_update(I, E, conv.dimF, (0, 1, 1), (1, 1, 1), 0.25)
+        scale = np.abs(ref).mean()
+        for late, shuffle in MODES:
+            got = conv.update(I, E, alpha=0.25, late_loads=late, shuffle=shuffle, cus=cus)
+            err = np.abs(got - ref).max() / scale
+            assert err < 2e-5, ("strips", (N, C, K, H, W, cus, late), err)
+
+
 if __name__ == "__main__":
-    {"fc": fc, "nt": nt, "rows": rows}[sys.argv[1]]()
+    {"fc": fc, "nt": nt, "rows": rows, "strips": strips}[sys.argv[1]]()
     print("ok", sys.argv[1])

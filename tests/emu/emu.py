@@ -122,8 +122,8 @@ class Conv(object):
         lib.ng_conv_plan_workspace_bytes.argtypes = [c_void_p]
         self.ws_bytes = lib.ng_conv_plan_workspace_bytes(self.plan)
 
-    def _run(self, call, tensors, late_loads, shuffle):
-        lib = _configure(8, late_loads, shuffle)
+    def _run(self, call, tensors, late_loads, shuffle, cus=8):
+        lib = _configure(cus, late_loads, shuffle)
         ws = aligned((max(self.ws_bytes, 16),), np.uint8, 0xAB)
         bufs = list(tensors) + [ws]
         for b in bufs:
@@ -156,14 +156,14 @@ class Conv(object):
         self._run(call, (dF, dE, dB), late_loads, shuffle)
         return np.array(dB)
 
-    def update(self, I, E, alpha=1.0, late_loads=False, shuffle=0):
+    def update(self, I, E, alpha=1.0, late_loads=False, shuffle=0, cus=8, workspace=True):
         dI, dE = aligned(I.shape, I.dtype, I), aligned(E.shape, E.dtype, E)
         dU = aligned(self.dimF, np.float32, 7)
         def call(lib, ws):
             lib.ng_conv_update.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_size_t, c_void_p]
             return lib.ng_conv_update(self.plan, self.code, NG_F32, dI.ctypes.data, dE.ctypes.data, dU.ctypes.data, alpha,
-                                      ws.ctypes.data, self.ws_bytes, None)
-        self._run(call, (dI, dE, dU), late_loads, shuffle)
+                                      ws.ctypes.data if workspace else None, self.ws_bytes if workspace else 0, None)
+        self._run(call, (dI, dE, dU), late_loads, shuffle, cus)
         return np.array(dU)
 
 

@@ -129,14 +129,15 @@ def test_emulated_pooling(emu, case):
 
 CANDIDATES = [("fc", {"NG_FC_CFG": "1"}), ("fc", {"NG_FC_CFG": "2"}), ("fc", {"NG_FC_CFG": "3"}),
               ("fc", {"NG_FC_CFG": "7"}), ("fc", {"NG_FC_CFG": "8"}),
-              ("nt", {"NG_NT_STREAM": "1"}), ("nt", {"NG_NT_STREAM": "2"}), ("rows", {"NG_CONV_ROWS": "1"})]
+              ("nt", {"NG_NT_STREAM": "1"}), ("nt", {"NG_NT_STREAM": "2"}), ("rows", {"NG_CONV_ROWS": "1"}),
+              ("strips", {"NG_UPDATE_STRIPS": "1"})]
 
 
 @pytest.mark.parametrize("what,switch", CANDIDATES)
 def test_emulated_candidate_kernels(emu, what, switch):
     """kernels that wait behind environment switches for their first measurement on a device
     (tests/emu/candidates.py): split k-steps inside a workgroup, the streamed outer-product GEMM,
-    the first-layer forward with decoded taps"""
+    the first-layer forward with decoded taps, the weight gradient on strips"""
     env = dict(os.environ)
     env.update(switch)
     done = subprocess.run([sys.executable, os.path.join(os.path.dirname(os.path.abspath(__file__)), "emu", "candidates.py"), what],
