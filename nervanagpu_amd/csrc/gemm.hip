@@ -219,6 +219,9 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
             // the same rows without the in-workgroup split: a whole CU of LDS as stages of the weight stream
             case 8: return launch_layout<_Float16, 128, 128, 32, 2, 2, true, 8, 1, true>(g, sr_bits);
             case 9: return launch_layout<_Float16, 128, 128, 64, 2, 2, true, 4, 1, true>(g, sr_bits);
+            // 64 rows (half the slices, i.e. half the partial sums, of 128) with six stages: 40 KB of weights in flight
+            case 11: return launch_layout<_Float16, 64, 128, 64, 2, 2, true, 6, 1, true>(g, sr_bits);
+            case 12: return launch_layout<_Float16, 64, 128, 64, 2, 1, true, 6, 2>(g, sr_bits);
             default: break;
             }
         }
