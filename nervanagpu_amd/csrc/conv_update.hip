@@ -115,12 +115,12 @@ static int launch_update_strip(const ConvPlan& pl, const void* I, const void* E,
     s.tiles_m = 1; s.tiles_n = 1;
     s.passes = 1;
     const int strips = cdiv(p.W, WT);
-    const int steps = strips * (p.H + 2) * (WT + 2);
-    s.k_tiles = steps;
+    const int strip_rows = strips * (p.H + 2);      // the unit of a contraction slice: WT + 2 steps each
+    s.k_tiles = strip_rows;
     const size_t slice = (size_t)rows * cols * sizeof(float);
-    s.splits = ws ? conv_splits(1, steps, slice, ws_bytes, 1) : 1;
+    s.splits = ws ? conv_splits(1, strip_rows, slice, ws_bytes, 1) : 1;
     UpdateStripGeom g{(const _Float16*)I, (const _Float16*)E, p.C, p.K, p.H, p.W, strips, p.H * p.W * p.N,
-                      p.P * p.Q * p.N, steps, FastDiv::make((unsigned)(WT + 2)), FastDiv::make((unsigned)(p.H + 2))};
+                      p.P * p.Q * p.N, strip_rows, FastDiv::make((unsigned)(p.H + 2))};
     ScaleStoreEpilogue<TOUT> epi{(TOUT*)gradF, 0, p.K, rows, cols, alpha, 0.0f, 0u, 0u, 0u, 0u,
                                  (((uintptr_t)gradF & 15) == 0) ? 1u : 0u};
     const dim3 grid(grid_tiles(1, s.splits), grid_slices(1, s.splits), 1);

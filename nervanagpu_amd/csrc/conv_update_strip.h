@@ -13,14 +13,19 @@
 // Every input pixel of the strip (WT + 2 columns wide, so strips overlap by two) is
 // requested once.
 //
-// Walk: a strip has WS = WT + 2 positions per row and H + 2 rows yy = -2 .. H-1 (the two
-// rows before the image fill the ring; their steps multiply nothing).  Position
-// p = (strip * (H + 2) + yy + 2) * WS + xs.  The A stream holds input pixel
+// Walk: a strip has H + 2 rows yy = -2 .. H-1 (the two rows before the image fill the
+// ring; their steps multiply nothing) of WS = WT + 2 positions xs.  Strip row
+// gr = strip * (H + 2) + yy + 2, position p = gr * WS + xs.  The A stream holds input pixel
 // (row yy + 1, column x0 + xs - 1) at position p (rows -1 and H and columns -1 and W are
 // the zero padding); the B stream holds output pixel (yy, x0 + xs) for yy >= 0, xs < WT
 // (else nothing: the step only moves the ring).  Tap (r,s) of step p reads A position
-// p + s - (2 - r) * WS.  A contraction slice is a range of positions; its first
-// 2 * WS + 2 requests refill the ring.
+// p + s - (2 - r) * WS.  A contraction slice is a range of strip rows; the loop starts three
+// rows early with the products switched off, which refills the ring.
+//
+// Everything that depends on the strip row (addresses, which positions exist) is decoded
+// once per row on the scalar unit into an offset and a bit mask per stream; the WS steps of
+// a row are unrolled, so what depends on xs is a compile-time constant: twelve wavefronts
+// repeat the scalar part of a step, and it has to stay well below the 12 MFMAs of the step.
 #pragma once
 #include "conv_plan.h"
 
@@ -34,8 +39,8 @@ struct UpdateStripGeom {
     int strips;         // ceil(W / WT)
     int chan_stride;    // elements between channels of I: H*W*N
     int kdim;           // row length of E: H*W*N
-    int steps;          // strips * (H + 2) * WS
-    FastDiv ws_div, rows_div;   // by WS, by H + 2
+    int rows;           // strip rows: strips * (H + 2)
+    FastDiv rows_div;   // by H + 2
 };
 
 // WT output columns per strip; LEAD: steps a request is issued ahead of its use
@@ -48,8 +53,11 @@ void conv_update_strip_kernel(UpdateStripGeom g, Epi epi, CoreShape s)
     constexpr int N = 64;                          // images per pixel = contraction elements per step
     constexpr int CB = 64, BN = 64;                // channels (rows of a slot), output maps
     constexpr int WS = WT + 2, TAPS = 3;
-    constexpr int WM = 6, WN = 2, NT = WM * WN * 64;   // wavefront rows: (channel block, vertical tap)
+    constexpr int WM = 6, WN = 2;                  // wavefront rows: (channel block, vertical tap)
+    constexpr int A_LEAD = 2 + LEAD;               // positions the A stream runs ahead of the step
     constexpr int RING = 2 * WS + TAPS + LEAD, BST = 1 + LEAD;
+    static_assert(WS % BST == 0, "the stage of E of a step is a constant of its xs");
+    static_assert(A_LEAD < WS, "requests reach into the next strip row at most");
     using TA = SwizzledTile<T, KC, CB, N>;         // one input pixel: 64 channels x 128 bytes
     using TB = SwizzledTile<T, KC, BN, N>;         // one pixel of E: 64 maps x 128 bytes
     using FA = SwizzledFrag<KC, TA>;
@@ -71,72 +79,50 @@ void conv_update_strip_kernel(UpdateStripGeom g, Epi epi, CoreShape s)
 
     int tm, tn, split;
     if (!block_work(s, tm, tn, split)) return;
-    const int per = (g.steps + s.splits - 1) / s.splits;
-    const int i_begin = split * per;
-    const int i_end = min(i_begin + per, g.steps);
-    const int nsteps = i_end - i_begin;
+    const int per = (g.rows + s.splits - 1) / s.splits;
+    const int r_begin = split * per;
+    const int r_end = min(r_begin + per, g.rows);
 
     // wavefronts 0..7 request the input pixel (one chunk a lane), 8..11 the pixel of E (two)
     const bool loads_a = wave < 8;
-    int a_chan = 0;          // what of the address does not move with the walk
+    unsigned a_lane = 0;     // lane part of the byte offset: channel and image chunk
     bool a_valid = false;
-    unsigned b_off[2] = {NG_OOB_OFFSET, NG_OOB_OFFSET};
+    unsigned b_lane[2] = {NG_OOB_OFFSET, NG_OOB_OFFSET};
     if (loads_a) {
         int r, k;
         TA::chunk_pos(tid, r, k);
         a_valid = r < g.C;
-        a_chan = min(r, g.C - 1) * g.chan_stride + k;
+        a_lane = (unsigned)(min(r, g.C - 1) * g.chan_stride + k) * 2u;
     } else {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            const int chunk = (tid - 512) + i * 256;
             int r, k;
-            TB::chunk_pos(chunk, r, k);
-            b_off[i] = (r < g.K) ? ((unsigned)r * (unsigned)g.kdim + (unsigned)k) * 2u : NG_OOB_OFFSET;
+            TB::chunk_pos((tid - 512) + i * 256, r, k);
+            b_lane[i] = (r < g.K) ? ((unsigned)r * (unsigned)g.kdim + (unsigned)k) * 2u : NG_OOB_OFFSET;
         }
     }
     const BufferRsrc a_rsrc = make_rsrc(g.I), b_rsrc = make_rsrc(g.E);
 
-    // walkers (wavefront-uniform).  A: next position to request; starts 2 * WS positions before the slice
-    struct Walk { int strip, yy, xs; };
-    auto walk_at = [&](int p) {
-        Walk w;
-        if (p < 0) { w.strip = -1; w.yy = -2; w.xs = p; return w; }     // before the first strip: nothing
-        const int row = (int)g.ws_div.div((unsigned)p);
-        w.xs = p - row * WS;
-        w.strip = (int)g.rows_div.div((unsigned)row);
-        w.yy = row - w.strip * (g.H + 2) - 2;
-        return w;
-    };
-    auto advance = [&](Walk& w) {
-        if (w.strip < 0) { if (++w.xs == 0) { w.strip = 0; w.yy = -2; } return; }
-        if (++w.xs == WS) { w.xs = 0; if (++w.yy == g.H) { w.yy = -2; w.strip++; } }
-    };
-    Walk aw = walk_at(i_begin - 2 * WS), bw = walk_at(i_begin), cw = bw;
-
-    auto issue_a = [&](int slot) {
-        if (loads_a) {
-            const int row = aw.yy + 1, col = aw.strip * WT + aw.xs - 1;
-            const bool ok = a_valid & (aw.strip >= 0) & (aw.strip < g.strips) & ((unsigned)row < (unsigned)g.H) &
-                            ((unsigned)col < (unsigned)g.W);
-            const unsigned off = ok ? (unsigned)(a_chan + (row * g.W + col) * N) * 2u : NG_OOB_OFFSET;
-            buffer_load_chunk_to_lds(a_rsrc, smem + slot * TA::BYTES + (wave * 64) * 16, off);
+    // one strip row, decoded on the scalar unit: byte offset of position xs = 0 and the
+    // positions that exist, for the A stream (input pixels) and the B stream (pixels of E)
+    struct Row { unsigned a_off, a_mask, b_off, b_mask; };
+    auto decode = [&](int gr) {
+        Row r{0u, 0u, 0u, 0u};
+        if (gr < 0 || gr >= g.rows) return r;
+        const int st = (int)g.rows_div.div((unsigned)gr);
+        const int yy = gr - st * (g.H + 2) - 2;
+        const int x0 = st * WT;
+        if ((unsigned)(yy + 1) < (unsigned)g.H) {
+            // column x0 - 1 + xs: not before the image (strip 0, xs = 0), not past it
+            const int hi = min(WS, g.W - x0 + 1);
+            r.a_mask = ((1u << hi) - 1u) & (x0 == 0 ? ~1u : ~0u);
+            r.a_off = (unsigned)(((yy + 1) * g.W + x0 - 1) * N) * 2u;      // of xs = 0; wraps below zero for x0 = 0, where xs = 0 is masked
         }
-        advance(aw);
-    };
-    auto issue_b = [&](int stage) {
-        if (!loads_a) {
-            const int q = bw.strip * WT + bw.xs;
-            const bool ok = (bw.strip < g.strips) & (bw.yy >= 0) & (bw.xs < WT) & (q < g.W);
-            const unsigned pix = (unsigned)(bw.yy * g.W + q) * (unsigned)(N * 2);
-#pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const unsigned off = (ok & (b_off[i] != NG_OOB_OFFSET)) ? b_off[i] + pix : NG_OOB_OFFSET;
-                // chunk (wave - 8) * 64 + lane + i * 256: the hardware adds 16 * lane to the wavefront's base
-                buffer_load_chunk_to_lds(b_rsrc, smem + A_BYTES + stage * TB::BYTES + ((i * 4 + (wave - 8)) * 64) * 16, off);
-            }
+        if (yy >= 0 && gr >= r_begin && gr < r_end) {
+            r.b_mask = (1u << min(WT, g.W - x0)) - 1u;
+            r.b_off = (unsigned)((yy * g.W + x0) * N) * 2u;
         }
-        advance(bw);
+        return r;
     };
 
     float16_t acc[TAPS][1];
@@ -148,56 +134,64 @@ void conv_update_strip_kernel(UpdateStripGeom g, Epi epi, CoreShape s)
     const int fa_base = FA::base(cb, lane);
     const int fb_base = FB::base(wn, lane);
 
-    // slot / stage indices advance by counters (the ring lengths are not powers of two)
-    auto next = [](int v, int n) { return v + 1 == n ? 0 : v + 1; };
-    int a_wr = 0, b_wr = 0;         // where the next requests go
-    // slot of A position (step + s - (2 - rtap) * WS) for s = 0: the ring starts at position i_begin - 2 * WS
-    int a_rd = rtap * WS, b_rd = 0;
-    int issued = 0;                 // steps whose B request (and A request of position + 2) are out
-    auto issue_step = [&]() {
-        issue_a(a_wr); a_wr = next(a_wr, RING);
-        issue_b(b_wr); b_wr = next(b_wr, BST);
-        issued++;
-    };
-    if (nsteps > 0) {
-        // refill: A positions i_begin - 2 * WS .. i_begin + 1, then LEAD whole steps
-#pragma unroll 1
-        for (int l = 0; l < 2 * WS + 2; l++) { issue_a(a_wr); a_wr = next(a_wr, RING); }
+    // Ring slots as byte offsets.  The first request (made at the first step, for the position
+    // A_LEAD ahead) goes to slot 0, so the slot of tap (rtap, 0) of the first step is
+    // -A_LEAD - (2 - rtap) * WS modulo the ring; it only matters once real rows are multiplied.
+    auto wrap = [](int off) { return off + TA::BYTES == A_BYTES ? 0 : off + TA::BYTES; };
+    int a_wr = 0;
+    int rd0 = (((-A_LEAD - (2 - rtap) * WS) % RING + RING) % RING) * TA::BYTES;
+    int rd1 = wrap(rd0), rd2 = wrap(rd1);
+
+    Row cur = decode(r_begin - 3);
+    for (int gr = r_begin - 3; gr < r_end; gr++) {
+        const Row nxt = decode(gr + 1);
 #pragma unroll
-        for (int l = 0; l < LEAD; l++)
-            if (issued < nsteps) issue_step();
-    }
-    for (int j = 0; j < nsteps; j++) {
-        // the requests of step j have landed (those of later steps may still be in flight:
-        // vector-memory operations complete in issue order), and nobody still reads what the
-        // next requests overwrite (the oldest slot, the stage of step j-1)
-        if (LEAD > 1 && issued - j - 1 >= LEAD - 1) {
+        for (int xs = 0; xs < WS; xs++) {
+            // the requests of this step have landed (those of the next LEAD - 1 steps may still be in
+            // flight: vector-memory operations complete in issue order), and nobody still reads what
+            // the next requests overwrite (the oldest slot, the stage of the previous step)
             if (loads_a) __builtin_amdgcn_s_waitcnt(WaitVmLgkm0<(LEAD - 1) * 1>::IMM);
             else         __builtin_amdgcn_s_waitcnt(WaitVmLgkm0<(LEAD - 1) * 2>::IMM);
-        } else {
-            __builtin_amdgcn_s_waitcnt(WaitVmLgkm0<0>::IMM);
-        }
-        __syncthreads();
-        if (issued < nsteps) issue_step();
-        const bool multiply = (cw.strip < g.strips) & (cw.yy >= 0) & (cw.xs < WT) & (cw.strip * WT + cw.xs < g.W);
-        if (multiply) {
-            const char* bt = smem + A_BYTES + b_rd * TB::BYTES;
-            const int a1 = next(a_rd, RING), a2 = next(a1, RING);
-            const char* at[TAPS] = {smem + a_rd * TA::BYTES, smem + a1 * TA::BYTES, smem + a2 * TA::BYTES};
+            __syncthreads();
+            if (loads_a) {
+                const int xa = (xs + A_LEAD) % WS;       // constants once the loop is unrolled
+                const Row& r = (xs + A_LEAD < WS) ? cur : nxt;
+                const bool ok = (r.a_mask >> xa) & 1u;
+                const unsigned off = (ok & a_valid) ? a_lane + r.a_off + (unsigned)(xa * N * 2) : NG_OOB_OFFSET;
+                buffer_load_chunk_to_lds(a_rsrc, smem + a_wr + (wave * 64) * 16, off);
+            } else {
+                const int xb = (xs + LEAD) % WS;
+                const Row& r = (xs + LEAD < WS) ? cur : nxt;
+                const bool ok = (r.b_mask >> xb) & 1u;
+                const unsigned pix = r.b_off + (unsigned)(xb * N * 2);
 #pragma unroll
-            for (int kk = 0; kk < N / 16; kk++) {
-                const Frag<T> b = FB::load(bt, fb_base, kk);
-#pragma unroll
-                for (int t = 0; t < TAPS; t++) {
-                    const Frag<T> a = FA::load(at[t], fa_base, kk);
-                    mfma_step(a, b, acc[t][0]);
+                for (int i = 0; i < 2; i++) {
+                    const unsigned off = (ok & (b_lane[i] != NG_OOB_OFFSET)) ? b_lane[i] + pix : NG_OOB_OFFSET;
+                    // chunk (wave - 8) * 64 + lane + i * 256: the hardware adds 16 * lane to the wavefront's base
+                    buffer_load_chunk_to_lds(b_rsrc, smem + A_BYTES + (xb % BST) * TB::BYTES + ((i * 4 + (wave - 8)) * 64) * 16, off);
                 }
             }
+            a_wr = wrap(a_wr);
+            if ((cur.b_mask >> xs) & 1u) {
+                const char* bt = smem + A_BYTES + (xs % BST) * TB::BYTES;
+                const char* at[TAPS] = {smem + rd0, smem + rd1, smem + rd2};
+#pragma unroll
+                for (int kk = 0; kk < N / 16; kk++) {
+                    const Frag<T> b = FB::load(bt, fb_base, kk);
+#pragma unroll
+                    for (int t = 0; t < TAPS; t++) {
+                        const Frag<T> a = FA::load(at[t], fa_base, kk);
+                        mfma_step(a, b, acc[t][0]);
+                    }
+                }
+            }
+            rd0 = rd1; rd1 = rd2; rd2 = wrap(rd2);
         }
-        a_rd = next(a_rd, RING); b_rd = next(b_rd, BST);
-        advance(cw);
+        cur = nxt;
     }
 
+    // requests of the last steps (positions past the slice) may still be landing in the ring
+    __builtin_amdgcn_s_waitcnt(WaitVmLgkm0<0>::IMM);
     __syncthreads();
     char* stage = smem + wave * EPI_BYTES;
     // band s of this wavefront holds filter rows ((cb * 32 + i) * 3 + rtap) * 3 + s
