@@ -43,6 +43,27 @@ def test_no_gpu_means_loud_failure():
         ng.empty((4, 4))
 
 
+def test_gemm_workspace_of_the_fully_connected_shapes_fits_the_static_scratch():
+    """ng_gemm_workspace_bytes is host arithmetic (no device: 256 CUs assumed).  The minibatch-wide shapes of the
+    benchmark (benchmarks/cublas.py:64-71) only fill the chip with their contraction cut into slices; the
+    partial sums of every schedule the dispatcher may pick must fit the 32 MiB array that ng_gemm_noalloc and
+    the nervana_* entry points use, and an outer product (k = 128) or a chip-filling square needs none."""
+    import ctypes
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    lib.ng_gemm_workspace_bytes.restype = ctypes.c_size_t
+    lib.ng_gemm_workspace_bytes.argtypes = [ctypes.c_int] * 8
+    lib.ng_gemm_static_scratch_bytes.restype = ctypes.c_size_t
+    cap = lib.ng_gemm_static_scratch_bytes()
+    assert cap == 32 << 20
+    for (M, K) in ((4096, 9216), (4096, 4096), (1000, 4096)):
+        for (ta, m, n, k) in ((0, M, 128, K), (1, K, 128, M)):
+            need = lib.ng_gemm_workspace_bytes(0, ta, 0, m, n, k, 1, 1)
+            assert 0 < need <= cap, (ta, m, n, k, need)
+            assert need % (m * n * 4) == 0 and need // (m * n * 4) >= 2      # whole fp32 slices, at least two
+        assert lib.ng_gemm_workspace_bytes(0, 0, 1, M, K, 128, 1, 1) == 0
+    assert lib.ng_gemm_workspace_bytes(0, 0, 0, 4096, 4096, 4096, 1, 1) == 0
+
+
 def fake(ng, shape, dtype=np.float16, addr=0x100000, **kw):
     return GPUTensor(ng, shape, dtype, gpudata=addr, **kw)
 
