@@ -204,7 +204,18 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
         // (read once per process) picks one; unset, the measured 64x128x64 tile on 2x2 wavefronts runs
         static const int fc_cfg = getenv("NG_FC_CFG") ? atoi(getenv("NG_FC_CFG")) : 0;
         if (g.n > 64 && g.batch_grid == 1 && k_tiles >= 8) {
-            switch (fc_cfg) {
+            int cfg = fc_cfg;
+            if (cfg < 0) {
+                // the rule the candidates would be used by, from what their designs predict (to be
+                // replaced by what the first measurement says): few rows of a row-major A on 32-row
+                // tiles; rows that 64-row tiles spread over at most a chip on those (half the partial
+                // sums of 128-row tiles); more rows on 128-row tiles
+                const int tiles64 = ceil_div(g.m, 64);
+                if (!g.trans_a && g.m <= 2048) cfg = 10;
+                else if (tiles64 <= cus / 2) cfg = 11;
+                else cfg = 9;
+            }
+            switch (cfg) {
             case 1: return launch_layout<_Float16, 128, 128, 64, 4, 1, true, 4, 2>(g, sr_bits);
             case 2: return launch_layout<_Float16, 64, 128, 128, 2, 1, true, 3, 4>(g, sr_bits);
             case 3: return launch_layout<_Float16, 128, 128, 128, 2, 1, true, 2, 4>(g, sr_bits);
