@@ -14,6 +14,7 @@
 // is read once instead of once per class.  No atomics, no zero fill, fp32
 // accumulation, one rounding.
 #include "conv_plan.h"
+#include <cstdlib>
 #include "conv_stream_taps.h"
 
 namespace ng {
@@ -105,7 +106,7 @@ static int run_bprop_merged(const ConvPlan& pl, const void* F, const void* E, vo
     }
 }
 
-template <typename T, bool BLOCKED, int BM, int BN, int BK, int WM, int WN>
+template <typename T, bool BLOCKED, int BM, int BN, int BK, int WM, int WN, int NSTAGE = 2>
 static int bprop_class(const ConvPlan& pl, const BpropClass& c, const void* F, const T* Fs, const void* E, void* gradI,
                        float alpha, const void* mask, hipStream_t stream, int col_begin = 0, int col_end = -1,
                        void* ws = nullptr, size_t ws_bytes = 0)
@@ -131,9 +132,9 @@ static int bprop_class(const ConvPlan& pl, const BpropClass& c, const void* F, c
                                    FastDiv::make((unsigned)std::max(c.taps, 1)), c.taps};
         // the filter is read in place, so the scratch is free for contraction slices of a small grid
         if (dense && col_begin == 0 && col_end < 0)
-            return launch_core_sliced<T, BM, BN, BK, WM, WN, KC, MC>(al, bl, depi, p.C, ncols, k_tiles, ws, ws_bytes, stream, "conv bprop");
-        if (dense) return launch_core<T, BM, BN, BK, WM, WN, KC, MC>(al, bl, depi, p.C, ncols, k_tiles, 1, stream, "conv bprop", col_begin, col_end);
-        return launch_core<T, BM, BN, BK, WM, WN, KC, MC>(al, bl, lepi, p.C, ncols, k_tiles, 1, stream, "conv bprop", col_begin, col_end);
+            return launch_core_sliced<T, BM, BN, BK, WM, WN, KC, MC, NSTAGE>(al, bl, depi, p.C, ncols, k_tiles, ws, ws_bytes, stream, "conv bprop");
+        if (dense) return launch_core<T, BM, BN, BK, WM, WN, KC, MC, NSTAGE>(al, bl, depi, p.C, ncols, k_tiles, 1, stream, "conv bprop", col_begin, col_end);
+        return launch_core<T, BM, BN, BK, WM, WN, KC, MC, NSTAGE>(al, bl, lepi, p.C, ncols, k_tiles, 1, stream, "conv bprop", col_begin, col_end);
     } else {
         DenseLoader<T, MC, true> al{Fs + c.w_row * pl.Cpad, 0, pl.Cpad, pl.Cpad, c.J};
         if (dense) return launch_core<T, BM, BN, BK, WM, WN, MC, MC>(al, bl, depi, p.C, ncols, k_tiles, 1, stream, "conv bprop", col_begin, col_end);
@@ -285,6 +286,14 @@ static int bprop_class_h(const ConvPlan& pl, const BpropClass& c, const void* F,
                                            : bprop_class<_Float16, BLOCKED, 128, 256, 64, 2, 4>(pl, c, F, Fs, E, gradI, alpha, mask, st, 0, cut);
             return rc ? rc : bprop_class<_Float16, BLOCKED, 64, 64, 64, 2, 2>(pl, c, F, Fs, E, gradI, alpha, mask, st, cut, -1);
         }
+    }
+    if constexpr (BLOCKED) {
+        // A candidate that has not been measured on a device yet (NG_CONV_STAGES=3, read once per process): a grid of
+        // at most one workgroup per CU has nobody to cover the wait for a tile requested one tile step ahead; a
+        // third stage (144 KB) gives the request two steps
+        static const int stages = getenv("NG_CONV_STAGES") ? atoi(getenv("NG_CONV_STAGES")) : 2;
+        if (stages == 3 && row_tile == 128 && (long)cdiv(pl.p.C, 128) * cdiv(ncols, 256) <= device_cu_count())
+            return bprop_class<_Float16, BLOCKED, 128, 256, 64, 2, 4, 3>(pl, c, F, Fs, E, gradI, alpha, mask, st, 0, -1, ws, ws_bytes);
     }
     switch (row_tile) {
     case 256: return bprop_class<_Float16, BLOCKED, 256, 256, 64, 2, 4>(pl, c, F, Fs, E, gradI, alpha, mask, st, 0, -1, ws, ws_bytes);

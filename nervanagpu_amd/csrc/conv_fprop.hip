@@ -285,6 +285,14 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
             return rc ? rc : fprop_tile<_Float16, TIN, BLOCKED, 64, 64, 64, 2, 2>(pl, I, F, O, alpha, flags, st, cut, -1);
         }
     }
+    if constexpr (BLOCKED && std::is_same<TIN, _Float16>::value) {
+        // A candidate that has not been measured on a device yet (NG_CONV_STAGES=3, read once per process): a grid of
+        // at most one workgroup per CU has nobody to cover the wait for a tile requested one tile step ahead; a
+        // third stage (144 KB) gives the request two steps
+        static const int stages = getenv("NG_CONV_STAGES") ? atoi(getenv("NG_CONV_STAGES")) : 2;
+        if (stages == 3 && row_tile == 128 && (long)cdiv(pl.p.K, 128) * cdiv(ncols, 256) <= device_cu_count())
+            return fprop_tile<_Float16, TIN, BLOCKED, 128, 256, 64, 2, 4, 3>(pl, I, F, O, alpha, flags, st, 0, -1, ws, ws_bytes);
+    }
     switch (row_tile) {
     case 256: return fprop_tile<_Float16, TIN, BLOCKED, 256, 256, 64, 2, 4>(pl, I, F, O, alpha, flags, st, 0, -1, ws, ws_bytes);
     // 128 rows on eight wavefronts: mid-sized layers run about one workgroup per

@@ -8,7 +8,10 @@ device (the switches are read once per process, hence this separate script):
     NG_UPDATE_STRIPS=1 weight gradient of 3x3 filters with at most 64 channels and output maps: strips of four
                        output columns, all nine taps on one ring of input pixels
 
-usage: python tests/emu/candidates.py fc|nt|rows|strips   (with the switch set in the environment)
+    NG_CONV_STAGES=3   forward / data gradient on 128x256x64 tiles of a grid of at most one workgroup per CU:
+                       three LDS stages
+
+usage: python tests/emu/candidates.py fc|nt|rows|strips|stages   (with the switch set in the environment)
 Every case runs with loads landing at once and with loads landing as late as the wait counts allow."""
 import os
 import sys
@@ -96,6 +99,21 @@ def strips():
             assert err < 2e-5, ("strips", (N, C, K, H, W, cus, late), err)
 
 
+def stages():
+    rng = np.random.default_rng(6)
+    # channels in blocks of 32, image rows that do not share taps (14 and 7 pixels), 128-row tiles, at most 8 column tiles
+    for (N, C, K, H, W) in [(64, 128, 128, 2, 14), (16, 160, 256, 7, 7)]:
+        conv = emu.Conv(np.float16, N, C, K, (1, H, W), (1, 3, 3), (0, 1, 1), (1, 1, 1))
+        I = rng.uniform(-1, 1, conv.dimI).astype(np.float16)
+        F = rng.uniform(-1, 1, conv.dimF).astype(np.float16)
+        E = rng.uniform(-1, 1, conv.dimO).astype(np.float16)
+        for late, shuffle in MODES:
+            O = conv.fprop(I, F, relu=True, late_loads=late, shuffle=shuffle)
+            assert_fp16_within_ulp(O, orc.ref_conv_fprop(I, F, (0, 1, 1), (1, 1, 1), 1.0, True), 1.0, "stages fprop", acc_atol(C * 9))
+            B = conv.bprop(F, E, late_loads=late, shuffle=shuffle)
+            assert_fp16_within_ulp(B, orc.ref_conv_bprop(F, E, conv.dimI, (0, 1, 1), (1, 1, 1)), 1.0, "stages bprop", acc_atol(K * 9))
+
+
 if __name__ == "__main__":
-    {"fc": fc, "nt": nt, "rows": rows, "strips": strips}[sys.argv[1]]()
+    {"fc": fc, "nt": nt, "rows": rows, "strips": strips, "stages": stages}[sys.argv[1]]()
     print("ok", sys.argv[1])

@@ -125,14 +125,14 @@ void vmem_wait(int outstanding)
     while ((int)q.size() > outstanding) { apply(q.front()); q.pop_front(); }
 }
 
-void launch(dim3 grid, dim3 block, const std::function<void()>& body)
+void launch(dim3 grid, dim3 block, const std::function<void()>& body, const char* name)
 {
     const int nthreads = (int)(block.x * block.y * block.z);
     const int nwaves = (nthreads + 63) / 64;
     g_grid = grid; g_block = block;
     g_body = &body;
     static const bool trace = std::getenv("EMU_TRACE") != nullptr;
-    if (trace) std::fprintf(stderr, "emu: launch grid (%u,%u,%u) block %u\n", grid.x, grid.y, grid.z, block.x);
+    if (trace) std::fprintf(stderr, "emu: launch grid (%u,%u,%u) block %u  %.400s\n", grid.x, grid.y, grid.z, block.x, name ? name : "");
     std::mt19937 rng(g_shuffle_seed);
     std::vector<int> order(nthreads);
     for (unsigned bz = 0; bz < grid.z; bz++)

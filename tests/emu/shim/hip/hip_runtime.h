@@ -72,7 +72,7 @@ void wg_sync();                   // __syncthreads
 // (64 bytes each) of this rendezvous: write your own before, read any after
 char* wave_exchange_begin();      // slots to deposit into
 void wave_exchange_sync();        // all lanes have deposited
-void launch(dim3 grid, dim3 block, const std::function<void()>& body);
+void launch(dim3 grid, dim3 block, const std::function<void()>& body, const char* name = nullptr);
 
 // vector-memory operations of the current wavefront that s_waitcnt vmcnt counts
 void vmem_issue(char* lds_dst, const void* src16);   // 16 bytes to LDS (src16 == nullptr: zeros)
@@ -86,7 +86,7 @@ void vmem_wait(int outstanding);
 #define gridDim (emu::g_grid)
 #define blockDim (emu::g_block)
 #define hipLaunchKernelGGL(kernel, grid, block, shmem, stream, ...) \
-    emu::launch((grid), (block), [=]() { kernel(__VA_ARGS__); })
+    emu::launch((grid), (block), [=]() { kernel(__VA_ARGS__); }, __PRETTY_FUNCTION__)
 
 inline void __syncthreads() { emu::wg_sync(); }
 

@@ -130,7 +130,7 @@ def test_emulated_pooling(emu, case):
 CANDIDATES = [("fc", {"NG_FC_CFG": "1"}), ("fc", {"NG_FC_CFG": "2"}), ("fc", {"NG_FC_CFG": "3"}),
               ("fc", {"NG_FC_CFG": "7"}), ("fc", {"NG_FC_CFG": "8"}),
               ("nt", {"NG_NT_STREAM": "1"}), ("nt", {"NG_NT_STREAM": "2"}), ("rows", {"NG_CONV_ROWS": "1"}),
-              ("strips", {"NG_UPDATE_STRIPS": "1"})]
+              ("strips", {"NG_UPDATE_STRIPS": "1"}), ("stages", {"NG_CONV_STAGES": "3"})]
 
 
 @pytest.mark.parametrize("what,switch", CANDIDATES)
