@@ -288,11 +288,10 @@ static int bprop_class_h(const ConvPlan& pl, const BpropClass& c, const void* F,
         }
     }
     if constexpr (BLOCKED) {
-        // A candidate that has not been measured on a device yet (NG_CONV_STAGES=3, read once per process): a grid of
-        // at most one workgroup per CU has nobody to cover the wait for a tile requested one tile step ahead; a
-        // third stage (144 KB) gives the request two steps
-        static const int stages = getenv("NG_CONV_STAGES") ? atoi(getenv("NG_CONV_STAGES")) : 2;
-        if (stages == 3 && row_tile == 128 && (long)cdiv(pl.p.C, 128) * cdiv(ncols, 256) <= device_cu_count())
+        // A candidate that has not been measured on a device yet (conv_stage_switch): a grid of at most one
+        // workgroup per CU has nobody to cover the wait for a tile requested one tile step ahead; a third
+        // stage (144 KB) gives the request two steps
+        if (conv_stage_switch() >= 3 && row_tile == 128 && (long)cdiv(pl.p.C, 128) * cdiv(ncols, 256) <= device_cu_count())
             return bprop_class<_Float16, BLOCKED, 128, 256, 64, 2, 4, 3>(pl, c, F, Fs, E, gradI, alpha, mask, st, 0, -1, ws, ws_bytes);
     }
     switch (row_tile) {
@@ -335,8 +334,10 @@ static int run_bprop(const ConvPlan& pl, const void* F, const void* E, void* gra
             // padded image rows can cost a round over the chip more than the separate taps need
             double cost, cost_plain;
             const int row_tile = pick_row_tile(p.C, p.D * p.H * cdiv(p.W, 2) * 2 * p.N, 256, &cost);
-            pick_row_tile(p.C, p.D * p.H * p.W * p.N, 256, &cost_plain);
-            if (cost <= cost_plain && row_tile >= 128) {
+            const int plain_tile = pick_row_tile(p.C, p.D * p.H * p.W * p.N, 256, &cost_plain);
+            const bool three_stages = conv_stage_switch() == 4 && plain_tile == 128 && blocked &&
+                                      (long)cdiv(p.C, 128) * cdiv(p.D * p.H * p.W * p.N, 256) <= device_cu_count();
+            if (cost <= cost_plain && row_tile >= 128 && !three_stages) {
                 const int ncols = p.D * p.H * cdiv(p.W, 2) * 2 * p.N;
                 const int tail = tail_column_tiles(cdiv(p.C, row_tile), cdiv(ncols, 256));
                 const int cut = tail ? (cdiv(ncols, 256) - tail) * 256 : -1;

@@ -193,8 +193,11 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
             // than the unpadded columns of the separate taps need: not worth it then
             double cost, cost_plain;
             const int row_tile = pick_row_tile(pl.p.K, ncols, 256, &cost);
-            pick_row_tile(pl.p.K, pl.p.M * pl.p.P * pl.p.Q * pl.p.N, 256, &cost_plain);
-            if (cost <= cost_plain && row_tile >= 128) {
+            const int plain_cols = pl.p.M * pl.p.P * pl.p.Q * pl.p.N;
+            const int plain_tile = pick_row_tile(pl.p.K, plain_cols, 256, &cost_plain);
+            const bool three_stages = conv_stage_switch() == 4 && plain_tile == 128 &&
+                                      (long)cdiv(pl.p.K, 128) * cdiv(plain_cols, 256) <= device_cu_count();
+            if (cost <= cost_plain && row_tile >= 128 && !three_stages) {
                 // trailing column tiles beyond whole rounds: 64-row tiles of one pixel behind the main launch
                 const int tail = tail_column_tiles(cdiv(pl.p.K, row_tile), cdiv(ncols, 256));
                 const int cut = tail ? (cdiv(ncols, 256) - tail) * 256 : -1;
@@ -286,11 +289,10 @@ static int fprop_h(const ConvPlan& pl, const void* I, const void* F, void* O, fl
         }
     }
     if constexpr (BLOCKED && std::is_same<TIN, _Float16>::value) {
-        // A candidate that has not been measured on a device yet (NG_CONV_STAGES=3, read once per process): a grid of
-        // at most one workgroup per CU has nobody to cover the wait for a tile requested one tile step ahead; a
-        // third stage (144 KB) gives the request two steps
-        static const int stages = getenv("NG_CONV_STAGES") ? atoi(getenv("NG_CONV_STAGES")) : 2;
-        if (stages == 3 && row_tile == 128 && (long)cdiv(pl.p.K, 128) * cdiv(ncols, 256) <= device_cu_count())
+        // A candidate that has not been measured on a device yet (conv_stage_switch): a grid of at most one
+        // workgroup per CU has nobody to cover the wait for a tile requested one tile step ahead; a third
+        // stage (144 KB) gives the request two steps
+        if (conv_stage_switch() >= 3 && row_tile == 128 && (long)cdiv(pl.p.K, 128) * cdiv(ncols, 256) <= device_cu_count())
             return fprop_tile<_Float16, TIN, BLOCKED, 128, 256, 64, 2, 4, 3>(pl, I, F, O, alpha, flags, st, 0, -1, ws, ws_bytes);
     }
     switch (row_tile) {

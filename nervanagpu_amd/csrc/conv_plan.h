@@ -1,6 +1,7 @@
 // Host-side description of one convolution geometry, shared by the three
 // convolution translation units.
 #pragma once
+#include <cstdlib>
 
 #include "conv_loaders.h"
 #include "stream_core.h"
@@ -66,6 +67,16 @@ inline bool blocks_pay(int channels, int bk) { return channels % bk == 0 || 2 * 
 // round more (VGG weight gradients 7-22 % faster than with a rounded-up one and
 // a half per CU).  Contractions too short to leave 15 tiles per slice get one
 // workgroup per CU: the fp32 partials then cost more than the overlap gains.
+// NG_CONV_STAGES (read once per process), candidates that have not been measured on a device yet:
+// 3 = forward / data gradient grids of at most one workgroup per CU of 128x256x64 tiles run three
+// LDS stages; 4 = also, layers of 128 images on such grids leave the shared taps (whose 56 KB stages
+// only fit twice) for those tiles.  Unset: two stages everywhere, as measured.
+inline int conv_stage_switch()
+{
+    static const int v = std::getenv("NG_CONV_STAGES") ? std::atoi(std::getenv("NG_CONV_STAGES")) : 2;
+    return v;
+}
+
 inline int conv_splits(int out_tiles, int total_k_tiles, size_t slice_bytes, size_t ws_bytes, int per_cu = 2)
 {
     const int cus = device_cu_count();
