@@ -233,6 +233,8 @@ int dispatch<_Float16>(const GemmArgs& g, unsigned sr_bits)
             // 64 rows (half the slices, i.e. half the partial sums, of 128) with six stages: 40 KB of weights in flight
             case 11: return launch_layout<_Float16, 64, 128, 64, 2, 2, true, 6, 1, true>(g, sr_bits);
             case 12: return launch_layout<_Float16, 64, 128, 64, 2, 1, true, 6, 2>(g, sr_bits);
+            // the measured kernel and its slicing (one and a half workgroups per CU; two fit) with a third stage only
+            case 13: return launch_layout<_Float16, 64, 128, 64, 2, 2, true, 3>(g, sr_bits);
             default: break;
             }
         }

@@ -1,7 +1,7 @@
 """Checks of the candidate kernels that sit behind environment switches until they are measured on a
 device (the switches are read once per process, hence this separate script):
 
-    NG_FC_CFG=1..12    minibatch-wide GEMM: workgroups whose wavefront groups split the k-steps of a tile,
+    NG_FC_CFG=1..13    minibatch-wide GEMM: workgroups whose wavefront groups split the k-steps of a tile,
                        or that spend a whole CU of LDS on stages of the weight stream
     NG_NT_STREAM=1|2   outer-product GEMM: rows of A resident in registers, output columns streamed
     NG_CONV_ROWS=1     first-layer forward with large filters: taps decoded from the contraction row
